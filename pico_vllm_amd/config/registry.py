@@ -1,5 +1,5 @@
 """One registry from an architecture's name (``architectures[0]`` of
-config.json) to its typed configuration and its model description.
+config.json, or its ``architecture``) to its typed configuration and its model description.
 
 The reference has no registry: its entry script imports the one model class
 directly (pico_vllm/run_single.py:2,10-11).
@@ -37,6 +37,8 @@ def known_architectures():
 
 def resolve_architecture(raw_config: Dict[str, Any]) -> Architecture:
     names = raw_config.get("architectures")
+    if not names and isinstance(raw_config.get("architecture"), str):
+        names = [raw_config["architecture"]]
     if not names:
         raise ConfigError("config.json has no 'architectures' entry; known architectures: "
                           + ", ".join(known_architectures()))

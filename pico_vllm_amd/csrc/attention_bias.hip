@@ -1,0 +1,183 @@
+// Attention with a linear distance penalty, a query temperature that grows with the position, and keys and
+// values of different sizes, over the paged cache; and the store of its keys and values.
+//
+//   query head h reads kv head h / (nq / nkv)
+//   s_ij = (q_i . k_j) * scale * temp(i) - slope_h * (i - j),   keys j <= i, with a window only i - j < window
+//   temp(i) = 1 + coef * ln(floor((i + 1) / every) + 1)         (every == 0: 1)
+//   slope_h = 2^(-span * (h + 1) / nq)                          (span == 0: no penalty)
+//   softmax over the visible keys, o_i = sum_j p_ij v_j
+//
+// A page holds k as [kv heads, page, dk] and v as [kv heads, dv, page].  Scores, softmax and the sums over keys are
+// float32 whatever the storage type.  This file holds the plain kernel (one wave per query token and head, any sizes,
+// float32 or bfloat16 storage): the attention of the 32-bit engine and the fallback of the bfloat16 engine.
+#include "common.h"
+
+struct BiasParams {
+  float scale, temp_coef, slope_span;
+  int temp_every, window;
+};
+
+__device__ __forceinline__ float query_scale(const BiasParams& p, int pos) {
+  if (p.temp_every <= 0) return p.scale;
+  return p.scale * (1.0f + p.temp_coef * logf((float)((pos + 1) / p.temp_every + 1)));
+}
+
+__device__ __forceinline__ float head_slope(const BiasParams& p, int h, int nq) {
+  return p.slope_span > 0.f ? exp2f(-p.slope_span * (float)(h + 1) / (float)nq) : 0.f;
+}
+
+// ---------------------------------------------------------------------------
+// Store of a step's keys and values: token t's k and v (columns k_col.. and v_col.. of its row of `qkv`) go to slot
+// slots[t] (page * P + offset; negative: nothing is stored).  With `v_first` the value is mixed first:
+// v <- (1 - lambda) v + lambda v_first[t] in float32, and the mixed value is what the cache gets.
+// One workgroup per token.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void kv_mix_store_kernel(const T* __restrict__ qkv, int ld, int k_col, int v_col,
+                                                           const T* __restrict__ v_first, int ld_first, float lambda,
+                                                           const int* __restrict__ slots, T* __restrict__ k_cache,
+                                                           T* __restrict__ v_cache, int nkv, int dk, int dv, int P,
+                                                           int num_pages) {
+  const int t = blockIdx.x;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  const int page = slot / P, off = slot % P;
+  if (page >= num_pages) return;
+  const T* row = qkv + (size_t)t * ld;
+  for (int i = threadIdx.x; i < nkv * dk; i += blockDim.x) {
+    const int g = i / dk, j = i % dk;
+    k_cache[(((size_t)page * nkv + g) * P + off) * dk + j] = row[k_col + i];
+  }
+  for (int i = threadIdx.x; i < nkv * dv; i += blockDim.x) {
+    const int g = i / dv, j = i % dv;
+    T* dst = v_cache + (((size_t)page * nkv + g) * dv + j) * P + off;
+    if (v_first) {
+      const float v = load_f32(row + v_col + i), f = load_f32(v_first + (size_t)t * ld_first + i);
+      store_f32(dst, (1.0f - lambda) * v + lambda * f);
+    } else {
+      *dst = row[v_col + i];
+    }
+  }
+}
+
+extern "C" int pico_kv_mix_store(const void* qkv, int dtype, int ld, int k_col, int v_col, const void* v_first,
+                                 int ld_first, float lambda, const int* slots, void* k_cache, void* v_cache, int T,
+                                 int nkv, int dk, int dv, int P, int num_pages, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && nkv > 0 && dk > 0 && dv > 0 && P > 0 && num_pages > 0, "pico_kv_mix_store: bad sizes");
+  PICO_REQUIRE(k_col >= 0 && v_col >= 0 && ld >= k_col + nkv * dk && ld >= v_col + nkv * dv,
+               "pico_kv_mix_store: the row of %d columns does not hold the keys and values", ld);
+  PICO_REQUIRE(v_first == nullptr || ld_first >= nkv * dv, "pico_kv_mix_store: the rows of the first values are too short");
+  if (T == 0) return 0;
+  if (dtype == PICO_DTYPE_F32)
+    kv_mix_store_kernel<float><<<T, 256, 0, stream>>>((const float*)qkv, ld, k_col, v_col, (const float*)v_first, ld_first,
+                                                      lambda, slots, (float*)k_cache, (float*)v_cache, nkv, dk, dv, P,
+                                                      num_pages);
+  else if (dtype == PICO_DTYPE_BF16)
+    kv_mix_store_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)qkv, ld, k_col, v_col, (const bf16_t*)v_first,
+                                                       ld_first, lambda, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, nkv,
+                                                       dk, dv, P, num_pages);
+  else
+    PICO_REQUIRE(false, "pico_kv_mix_store: unknown dtype %d", dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The plain kernel.  Keys are visited in blocks of 64 aligned to absolute positions, so the result at a position does
+// not depend on how the sequence was cut into steps.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(64) void attn_bias_plain_kernel(
+    const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ positions,
+    const int* __restrict__ token_seq, T* __restrict__ out, int nq, int nkv, int dk, int dv, int P, BiasParams bp,
+    int num_pages) {
+  extern __shared__ float lds[];
+  float* qs = lds;        // [dk]
+  float* ps = lds + dk;   // [64]
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int g = h / (nq / nkv);
+  const int pos = positions[t];
+  const int* bt = block_table + (size_t)token_seq[t] * max_pages;
+  const int lo = bp.window > 0 ? max(0, pos - bp.window + 1) : 0;
+  const float qscale = query_scale(bp, pos), slope = head_slope(bp, h, nq);
+  const T* qrow = q + (size_t)t * q_stride + (size_t)h * dk;
+  for (int j = lane; j < dk; j += 64) qs[j] = load_f32(qrow + j);
+  __syncthreads();
+
+  float m = -INFINITY, l = 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int c0 = (lo / 64) * 64; c0 <= pos; c0 += 64) {
+    const int key = c0 + lane;
+    const bool valid = key >= lo && key <= pos;
+    float s = -INFINITY;
+    if (valid) {
+      int page = bt[key / P];
+      page = min(max(page, 0), num_pages - 1);
+      const T* kp = k_cache + (((size_t)page * nkv + g) * P + key % P) * dk;
+      float dot = 0.f;
+      for (int j = 0; j < dk; j++) dot = fmaf(qs[j], load_f32(kp + j), dot);
+      s = dot * qscale - slope * (float)(pos - key);
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float alpha = expf(m - m_new);
+    const float p = valid ? expf(s - m_new) : 0.f;
+    l = l * alpha + wave_sum(p);
+    __syncthreads();
+    ps[lane] = p;
+    __syncthreads();
+    float blk[4] = {0.f, 0.f, 0.f, 0.f};
+    const int kend = min(64, pos - c0 + 1);
+    for (int kk = max(0, lo - c0); kk < kend; kk++) {
+      const int kpos = c0 + kk;
+      int page = bt[kpos / P];
+      page = min(max(page, 0), num_pages - 1);
+      const T* vp = v_cache + ((size_t)page * nkv + g) * dv * P + kpos % P;
+      const float pk = ps[kk];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int dim = lane + 64 * i;
+        if (dim < dv) blk[i] = fmaf(pk, load_f32(vp + (size_t)dim * P), blk[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] = fmaf(acc[i], alpha, blk[i]);
+    m = m_new;
+  }
+  T* o = out + ((size_t)t * nq + h) * dv;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int dim = lane + 64 * i;
+    if (dim < dv) store_f32(o + dim, acc[i] / l);
+  }
+}
+
+extern "C" int pico_attn_bias_plain(const void* q, int q_stride, int dtype, const void* k_cache, const void* v_cache,
+                                    const int* block_table, int max_pages, const int* positions, const int* token_seq,
+                                    void* out, int T, int nq, int nkv, int dk, int dv, int P, int window, float scale,
+                                    float temp_coef, int temp_every, float slope_span, int num_pages,
+                                    hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && dk > 0 && dv > 0 && P > 0 && max_pages > 0 && num_pages > 0,
+               "pico_attn_bias_plain: bad sizes");
+  PICO_REQUIRE(nq % nkv == 0, "pico_attn_bias_plain: %d query heads are not a multiple of %d kv heads", nq, nkv);
+  PICO_REQUIRE(dk <= 1024 && dv <= 256, "pico_attn_bias_plain: key size %d (at most 1024) or value size %d (at most 256) too large", dk, dv);
+  PICO_REQUIRE(nq <= 65535, "pico_attn_bias_plain: too many heads");
+  PICO_REQUIRE(q_stride >= nq * dk, "pico_attn_bias_plain: query row stride too small");
+  PICO_REQUIRE(window >= 0 && temp_every >= 0 && slope_span >= 0.f, "pico_attn_bias_plain: window, interval and span must not be negative");
+  if (T == 0) return 0;
+  const BiasParams bp{scale, temp_coef, slope_span, temp_every, window};
+  dim3 grid(T, nq);
+  const size_t lds = (size_t)(dk + 64) * sizeof(float);
+  if (dtype == PICO_DTYPE_F32)
+    attn_bias_plain_kernel<float><<<grid, 64, lds, stream>>>(
+        (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, block_table, max_pages, positions,
+        token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages);
+  else if (dtype == PICO_DTYPE_BF16)
+    attn_bias_plain_kernel<bf16_t><<<grid, 64, lds, stream>>>(
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, positions,
+        token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages);
+  else
+    PICO_REQUIRE(false, "pico_attn_bias_plain: unknown dtype %d", dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}

@@ -467,3 +467,74 @@ extern "C" int pico_softcap(float* x, long long n, float cap, hipStream_t stream
   PICO_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// Learned rows added to the residual stream: resid[t, :] += table[idx[t], :] in float32 (absolute position
+// vectors: idx = the tokens' positions).  An index outside [0, N) adds nothing (the host refuses such a step).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void add_rows_kernel(float* __restrict__ resid, const T* __restrict__ table, const int* __restrict__ idx,
+                                int H, int N) {
+  const int t = blockIdx.x;
+  const int r = idx[t];
+  if (r < 0 || r >= N) return;
+  const T* row = table + (size_t)r * H;
+  float* o = resid + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] += load_f32(row + i);
+}
+
+extern "C" int pico_add_rows(float* resid, const void* table, int table_dtype, const int* idx, int T, int H, int N,
+                             hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && H > 0 && N > 0, "pico_add_rows: bad sizes T=%d H=%d N=%d", T, H, N);
+  if (T == 0) return 0;
+  if (table_dtype == PICO_DTYPE_F32)
+    add_rows_kernel<float><<<T, 256, 0, stream>>>(resid, (const float*)table, idx, H, N);
+  else if (table_dtype == PICO_DTYPE_BF16)
+    add_rows_kernel<bf16_t><<<T, 256, 0, stream>>>(resid, (const bf16_t*)table, idx, H, N);
+  else
+    PICO_REQUIRE(false, "pico_add_rows: unknown dtype %d", table_dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Squared ReLU: out = max(x, 0)^2, element by element (in place when out == x).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void relu2_kernel(const T* __restrict__ x, T* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) {
+    const float v = fmaxf(load_f32(x + i), 0.f);
+    store_f32(out + i, v * v);
+  }
+}
+
+__global__ void relu2_bf16x8_kernel(const uint4* __restrict__ x, uint4* __restrict__ out, size_t n8) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n8) return;
+  uint4 v = x[i];
+  uint32_t* w = reinterpret_cast<uint32_t*>(&v);
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const float a = fmaxf(__uint_as_float(w[j] << 16), 0.f), b = fmaxf(__uint_as_float(w[j] & 0xffff0000u), 0.f);
+    w[j] = pack2_bf16(a * a, b * b);
+  }
+  out[i] = v;
+}
+
+extern "C" int pico_relu2(const void* x, void* out, int dtype, long long n, hipStream_t stream) {
+  PICO_REQUIRE(n >= 0, "pico_relu2: bad size");
+  if (n == 0) return 0;
+  if (dtype == PICO_DTYPE_BF16 && n % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const size_t n8 = (size_t)n / 8;
+    relu2_bf16x8_kernel<<<(unsigned)((n8 + 255) / 256), 256, 0, stream>>>((const uint4*)x, (uint4*)out, n8);
+  } else if (dtype == PICO_DTYPE_BF16) {
+    relu2_kernel<bf16_t><<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, (size_t)n);
+  } else if (dtype == PICO_DTYPE_F32) {
+    relu2_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((const float*)x, (float*)out, (size_t)n);
+  } else {
+    PICO_REQUIRE(false, "pico_relu2: unknown dtype %d", dtype);
+  }
+  PICO_LAUNCH_CHECK();
+  return 0;
+}

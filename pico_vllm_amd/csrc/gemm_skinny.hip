@@ -50,6 +50,7 @@ struct TileRows {
 #define EPI_BF16 0     // out bf16 [M, N]
 #define EPI_F32 1      // out float32 [M, N] (slab `blockIdx.y` when the k range is split over the grid)
 #define EPI_SWIGLU 2   // W = [gate rows; up rows], out bf16 [M, N / 2]
+#define EPI_RELU2 3    // out bf16 [M, N] = max(x W^T + bias, 0)^2
 #define MAX_SK_SLABS 8 // partial sums that a norm in front of a projection adds up
 
 // The sums of one output tile when K is no multiple of 64 (any multiple of 8): operands go through
@@ -336,6 +337,10 @@ __device__ __forceinline__ void skinny_finish(float (*red)[MT][16][64], int tile
 #pragma unroll
         for (int w = 0; w < 4; w++) s += red[w][t][4 * a + b][lane];
         v[b] = s + ((bias && blockIdx.y == 0 && n + b < N) ? bias[n + b] : 0.f);
+        if (EPI == EPI_RELU2) {
+          v[b] = fmaxf(v[b], 0.f);
+          v[b] *= v[b];
+        }
       }
       if (EPI == EPI_F32) {
         float* o = (float*)out + (size_t)blockIdx.y * slab_stride + (size_t)m * ldo + n;
@@ -650,7 +655,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   PICO_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K,
                "pico_gemm_skinny: K and the row strides must be multiples of 8 (K=%d ldx=%d ldw=%d)", K, ldx, ldw);
   PICO_REQUIRE((uintptr_t)X % 16 == 0 && (uintptr_t)W % 16 == 0, "pico_gemm_skinny: operands must be 16-byte aligned");
-  PICO_REQUIRE(epilogue >= 0 && epilogue <= 2, "pico_gemm_skinny: unknown epilogue %d", epilogue);
+  PICO_REQUIRE(epilogue >= 0 && epilogue <= 3, "pico_gemm_skinny: unknown epilogue %d", epilogue);
   PICO_REQUIRE(k_splits >= 1 && (k_splits == 1 || epilogue == EPI_F32), "pico_gemm_skinny: only the float32 epilogue can split k over the grid");
   PICO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && bias == nullptr), "pico_gemm_skinny: SwiGLU needs an even N and no bias");
   const int n_out = epilogue == EPI_SWIGLU ? N / 2 : N;
@@ -681,6 +686,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   gemm_skinny_pair_kernel<EPI><<<pgrid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg, rows)
     if (epilogue == EPI_BF16) LAUNCHP(EPI_BF16);
     else if (epilogue == EPI_F32) LAUNCHP(EPI_F32);
+    else if (epilogue == EPI_RELU2) LAUNCHP(EPI_RELU2);
     else LAUNCHP(EPI_SWIGLU);
 #undef LAUNCHP
     PICO_LAUNCH_CHECK();
@@ -711,6 +717,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   } while (0)
   if (epilogue == EPI_BF16) LAUNCH(EPI_BF16);
   else if (epilogue == EPI_F32) LAUNCH(EPI_F32);
+  else if (epilogue == EPI_RELU2) LAUNCH(EPI_RELU2);
   else LAUNCH(EPI_SWIGLU);
 #undef LAUNCH4
 #undef LAUNCH

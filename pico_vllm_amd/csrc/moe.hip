@@ -1,0 +1,142 @@
+// A routed feed-forward (mixture of experts): the choice of experts and the experts' products.
+//
+//   scores s = sigmoid(z) of the router logits z (float32); a token's `top` experts are those with the largest z
+//   (the lowest index among equal ones), its weights their scores as they are
+//   expert e on a row x: g = min(Wg_e x, limit), u = clamp(Wu_e x, -limit, limit),
+//                        y = g * sigmoid(alpha g) * (u + 1), out = Wd_e y
+//   a token's output: sum over its experts of expert_e(w_e * x)     (the weight scales the expert's INPUT)
+//
+// Expert matrices are stacked: gate_up [E, 2 F, D] (an expert's gate rows, then its up rows), down [E, D, F].
+// This file holds the plain kernels (one wave per output element, any sizes, float32 or bfloat16 storage, every sum
+// in float32 and in an order that depends on the sizes alone); the matrix-core kernels for many rows stand behind them.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// Routing: one thread per token.
+// ---------------------------------------------------------------------------
+#define MOE_MAX_TOP 16
+
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int T, int E, int top,
+                                                       int* __restrict__ experts, float* __restrict__ weights) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* z = logits + (size_t)t * E;
+  int chosen[MOE_MAX_TOP];
+  for (int k = 0; k < top; k++) {
+    int best = -1;
+    float bz = 0.f;
+    for (int e = 0; e < E; e++) {
+      bool taken = false;
+      for (int j = 0; j < k; j++) taken |= chosen[j] == e;
+      if (taken) continue;
+      const float v = z[e];
+      if (best < 0 || v > bz) { best = e; bz = v; }     // NaN never wins over a number; the first of equals stays
+    }
+    chosen[k] = best;
+    experts[(size_t)t * top + k] = best;
+    weights[(size_t)t * top + k] = 1.0f / (1.0f + expf(-bz));
+  }
+}
+
+extern "C" int pico_moe_route(const float* logits, int T, int E, int top, int* experts, float* weights,
+                              hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E && top <= MOE_MAX_TOP,
+               "pico_moe_route: %d of %d experts per token is outside what the kernel takes (at most %d)", top, E, MOE_MAX_TOP);
+  if (T == 0) return 0;
+  moe_route_kernel<<<(T + 63) / 64, 64, 0, stream>>>(logits, T, E, top, experts, weights);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+__device__ __forceinline__ float expert_act(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+}
+
+// the input of an expert: the token's row times its weight, rounded to the storage type as a product's operand is
+template <typename T> __device__ __forceinline__ float scaled_input(const T* p, float w);
+template <> __device__ __forceinline__ float scaled_input<float>(const float* p, float w) { return *p * w; }
+template <> __device__ __forceinline__ float scaled_input<bf16_t>(const bf16_t* p, float w) {
+  return bf16_to_f32(f32_to_bf16(bf16_to_f32(*p) * w));
+}
+
+// ---------------------------------------------------------------------------
+// Plain first half: y[r, f] = act(gate_e[f] . x, up_e[f] . x) for row r = (token, slot), x = w_r * h[token].
+// grid (rows, ceil(F / 16)); four waves, each four outputs; the lanes of a wave split k.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void moe_up_plain_kernel(const T* __restrict__ h, int ldh, const T* __restrict__ gate_up,
+                                                           const int* __restrict__ experts, const float* __restrict__ weights,
+                                                           T* __restrict__ y, int top, int E, int F, int D, float limit,
+                                                           float alpha) {
+  const int r = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int e = experts[r];
+  if (e < 0 || e >= E) return;
+  const float w = weights[r];
+  const T* x = h + (size_t)(r / top) * ldh;
+  const T* We = gate_up + (size_t)e * 2 * F * D;
+  for (int i = 0; i < 4; i++) {
+    const int f = blockIdx.y * 16 + wave * 4 + i;
+    if (f >= F) break;
+    const T* wg = We + (size_t)f * D;
+    const T* wu = We + (size_t)(F + f) * D;
+    float g = 0.f, u = 0.f;
+    for (int j = lane; j < D; j += 64) {
+      const float xv = scaled_input<T>(x + j, w);
+      g = fmaf(load_f32(wg + j), xv, g);
+      u = fmaf(load_f32(wu + j), xv, u);
+    }
+    g = wave_sum(g);
+    u = wave_sum(u);
+    if (lane == 0) store_f32(y + (size_t)r * F + f, expert_act(g, u, limit, alpha));
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Plain second half: out[t, n] = sum over the token's slots (in slot order) of down_e[n] . y[(t, slot)], float32.
+// grid (tokens, ceil(D / 16)).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_plain_kernel(const T* __restrict__ y, const T* __restrict__ down,
+                                                             const int* __restrict__ experts, float* __restrict__ out,
+                                                             int top, int E, int F, int D) {
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int i = 0; i < 4; i++) {
+    const int n = blockIdx.y * 16 + wave * 4 + i;
+    if (n >= D) break;
+    float total = 0.f;
+    for (int k = 0; k < top; k++) {
+      const int r = t * top + k, e = experts[r];
+      if (e < 0 || e >= E) continue;
+      const T* wd = down + ((size_t)e * D + n) * F;
+      const T* yr = y + (size_t)r * F;
+      float s = 0.f;
+      for (int j = lane; j < F; j += 64) s = fmaf(load_f32(wd + j), load_f32(yr + j), s);
+      total += wave_sum(s);
+    }
+    if (lane == 0) out[(size_t)t * D + n] = total;
+  }
+}
+
+extern "C" int pico_moe_experts_plain(const void* h, int ldh, int dtype, const void* gate_up, const void* down,
+                                      const int* experts, const float* weights, void* y, float* out, int T, int top,
+                                      int E, int F, int D, float limit, float alpha, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && top > 0 && E > 0 && F > 0 && D > 0 && ldh >= D, "pico_moe_experts_plain: bad sizes");
+  if (T == 0) return 0;
+  const dim3 g1(T * top, (F + 15) / 16), g2(T, (D + 15) / 16);
+  PICO_REQUIRE(g1.y <= 65535 && g2.y <= 65535, "pico_moe_experts_plain: sizes beyond the grid");
+  if (dtype == PICO_DTYPE_F32) {
+    moe_up_plain_kernel<float><<<g1, 256, 0, stream>>>((const float*)h, ldh, (const float*)gate_up, experts, weights,
+                                                       (float*)y, top, E, F, D, limit, alpha);
+    moe_down_plain_kernel<float><<<g2, 256, 0, stream>>>((const float*)y, (const float*)down, experts, out, top, E, F, D);
+  } else if (dtype == PICO_DTYPE_BF16) {
+    moe_up_plain_kernel<bf16_t><<<g1, 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)gate_up, experts, weights,
+                                                        (bf16_t*)y, top, E, F, D, limit, alpha);
+    moe_down_plain_kernel<bf16_t><<<g2, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)down, experts, out, top, E, F, D);
+  } else {
+    PICO_REQUIRE(false, "pico_moe_experts_plain: unknown dtype %d", dtype);
+  }
+  PICO_LAUNCH_CHECK();
+  return 0;
+}

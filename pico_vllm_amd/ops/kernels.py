@@ -212,7 +212,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
     return out
 
 
-EPI_BF16, EPI_F32, EPI_SWIGLU = 0, 1, 2
+EPI_BF16, EPI_F32, EPI_SWIGLU, EPI_RELU2 = 0, 1, 2, 3
 MAX_HEAD_DIM = 256          # the largest head size any attention kernel takes
 
 
@@ -243,7 +243,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
                 k_splits: int = 1) -> torch.Tensor:
     """a [M <= 64, K] x w [N, K]^T, both bfloat16.  EPI_BF16 -> bf16 [M, N]; EPI_F32 -> float32 [M, N], or with
     k_splits > 1 a stack [k_splits, M, N] of partial sums (bias in the first); EPI_SWIGLU (w = [gate; up])
-    -> bf16 [M, N / 2] = silu(gate) * up."""
+    -> bf16 [M, N / 2] = silu(gate) * up; EPI_RELU2 -> bf16 [M, N] = max(x w^T + bias, 0)^2."""
     _gpu(a, w, bias)
     M, K = a.shape
     N, K2 = w.shape
@@ -525,4 +525,146 @@ def argmax(logits: torch.Tensor, out: torch.Tensor, work: tuple) -> torch.Tensor
             or not val.is_contiguous() or not idx.is_contiguous():
         raise KernelError("argmax: the workspace must come from argmax_workspace for at least as many rows")
     _check(lib, lib.pico_argmax(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(val), _ptr(idx), _ptr(out), _stream()))
+    return out
+
+
+def add_rows(resid: torch.Tensor, table: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+    """resid[t] += table[idx[t]] in float32, in place (learned position vectors: idx = positions)."""
+    _gpu(resid, table, idx)
+    T, H = resid.shape
+    if resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise KernelError("the residual stream must be contiguous float32")
+    if table.dim() != 2 or table.shape[1] != H or not table.is_contiguous():
+        raise KernelError(f"add_rows: the table must be contiguous [rows, {H}]")
+    _i32(idx, "idx", T)
+    lib = library.core()
+    _check(lib, lib.pico_add_rows(_ptr(resid), _ptr(table), _dt(table), _ptr(idx), T, H, table.shape[0], _stream()))
+    return resid
+
+
+def relu2(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """max(x, 0)^2 element by element (``out=x``: in place)."""
+    _gpu(x, out)
+    if not x.is_contiguous():
+        raise KernelError("relu2: the input must be contiguous")
+    if out is None:
+        out = torch.empty_like(x)
+    elif out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous():
+        raise KernelError("relu2: out has the wrong shape or dtype")
+    lib = library.core()
+    _check(lib, lib.pico_relu2(_ptr(x), _ptr(out), _dt(x), c_ll(x.numel()), _stream()))
+    return out
+
+
+def _check_cache2(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, dk: int, dv: int):
+    """K pages [pages, nkv, P, dk]; V pages [pages, nkv, dv, P]."""
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("cache tensors must be contiguous and 4-dimensional")
+    pages, h, P, dd = k_cache.shape
+    if (h, dd) != (nkv, dk) or tuple(v_cache.shape) != (pages, nkv, dv, P) or v_cache.dtype != k_cache.dtype:
+        raise KernelError(f"cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
+                          f"{nkv} kv heads with keys of {dk} and values of {dv}")
+    return pages, P
+
+
+def kv_mix_store(qkv: torch.Tensor, k_col: int, v_col: int, slots: torch.Tensor, k_cache: torch.Tensor,
+                 v_cache: torch.Tensor, nkv: int, dk: int, dv: int, v_first: Optional[torch.Tensor] = None,
+                 mix: float = 0.0) -> None:
+    """Write the keys (columns k_col ..) and values (columns v_col ..) of every row of ``qkv`` to ``slots`` (page * page
+    size + offset; negative: nothing).  With ``v_first`` [T, nkv * dv] (rows may be strided) the value stored is
+    (1 - mix) v + mix v_first, computed in float32."""
+    _gpu(qkv, slots, k_cache, v_cache, v_first)
+    T = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < max(k_col + nkv * dk, v_col + nkv * dv):
+        raise KernelError("kv_mix_store: qkv must be [T, columns] with unit stride along the row and hold keys and values")
+    pages, P = _check_cache2(k_cache, v_cache, nkv, dk, dv)
+    if k_cache.dtype != qkv.dtype:
+        raise KernelError("cache and activations differ in dtype")
+    _i32(slots, "slots", T)
+    if v_first is not None and (v_first.dtype != qkv.dtype or v_first.dim() != 2 or v_first.stride(1) != 1
+                                or tuple(v_first.shape) != (T, nkv * dv)):
+        raise KernelError(f"kv_mix_store: the first values must be [{T}, {nkv * dv}] of the activations' dtype")
+    lib = library.core()
+    _check(lib, lib.pico_kv_mix_store(_ptr(qkv), _dt(qkv), qkv.stride(0) if T > 1 else qkv.shape[1], k_col, v_col,
+                                      _ptr(v_first), 0 if v_first is None else (v_first.stride(0) if T > 1 else nkv * dv),
+                                      c_float(mix), _ptr(slots), _ptr(k_cache), _ptr(v_cache), T, nkv, dk, dv, P, pages,
+                                      _stream()))
+
+
+def attn_bias_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                    positions: torch.Tensor, token_seq: torch.Tensor, nq: int, nkv: int, dk: int, dv: int, scale: float,
+                    window: int = 0, temp_coef: float = 0.0, temp_every: int = 0, slope_span: float = 0.0,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention with a distance penalty slope_h (i - j), slope_h = 2^(-slope_span (h + 1) / nq), and the query
+    temperature 1 + temp_coef ln(floor((i + 1) / temp_every) + 1) on the scores.  q: [T, >= nq * dk]; returns [T, nq * dv]."""
+    _gpu(q, k_cache, v_cache, block_table, positions, token_seq)
+    T = q.shape[0]
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < nq * dk:
+        raise KernelError("q must be [T, >= nq*dk] with unit stride along the row")
+    pages, P = _check_cache2(k_cache, v_cache, nkv, dk, dv)
+    if k_cache.dtype != q.dtype:
+        raise KernelError("cache and activations differ in dtype")
+    _i32(positions, "positions", T)
+    _i32(token_seq, "token_seq", T)
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+        raise KernelError("block_table must be contiguous int32 [sequences, pages]")
+    if out is None:
+        out = torch.empty(T, nq * dv, dtype=q.dtype, device=q.device)
+    elif out.shape != (T, nq * dv) or out.dtype != q.dtype or not out.is_contiguous():
+        raise KernelError("attention: out has the wrong shape or dtype")
+    lib = library.core()
+    _check(lib, lib.pico_attn_bias_plain(_ptr(q), q.stride(0) if T > 1 else q.shape[1], _dt(q), _ptr(k_cache), _ptr(v_cache),
+                                         _ptr(block_table), block_table.shape[1], _ptr(positions), _ptr(token_seq), _ptr(out),
+                                         T, nq, nkv, dk, dv, P, window, c_float(scale), c_float(temp_coef), temp_every,
+                                         c_float(slope_span), pages, _stream()))
+    return out
+
+
+MOE_MAX_TOP = 16
+
+
+def moe_route(logits: torch.Tensor, top: int):
+    """(experts int32 [T, top], weights float32 [T, top]): every row's ``top`` largest logits (the lowest index among
+    equal ones) and their sigmoids."""
+    _gpu(logits)
+    T, E = logits.shape
+    if logits.dtype != torch.float32 or not logits.is_contiguous():
+        raise KernelError("moe_route: router logits must be contiguous float32")
+    if not 1 <= top <= min(E, MOE_MAX_TOP):
+        raise KernelError(f"moe_route: {top} of {E} experts per token (at most {MOE_MAX_TOP})")
+    experts = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    weights = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    lib = library.core()
+    _check(lib, lib.pico_moe_route(_ptr(logits), T, E, top, _ptr(experts), _ptr(weights), _stream()))
+    return experts, weights
+
+
+def _check_experts(h, gate_up, down, experts, weights, who):
+    T, D = h.shape
+    if gate_up.dim() != 3 or down.dim() != 3 or gate_up.shape[1] % 2:
+        raise KernelError(f"{who}: expert matrices are gate_up [E, 2 F, D] and down [E, D, F]")
+    E, F = gate_up.shape[0], gate_up.shape[1] // 2
+    if gate_up.shape[2] != D or tuple(down.shape) != (E, D, F) or not gate_up.is_contiguous() or not down.is_contiguous():
+        raise KernelError(f"{who}: expert matrices do not fit rows of {D}: {tuple(gate_up.shape)} / {tuple(down.shape)}")
+    if gate_up.dtype != h.dtype or down.dtype != h.dtype:
+        raise KernelError(f"{who}: activations and expert matrices differ in dtype")
+    if h.stride(1) != 1:
+        raise KernelError(f"{who}: activations must have unit stride along the row")
+    if experts.dtype != torch.int32 or weights.dtype != torch.float32 or experts.shape != weights.shape \
+            or experts.shape[0] != T or not experts.is_contiguous() or not weights.is_contiguous():
+        raise KernelError(f"{who}: experts int32 [T, top] and weights float32 [T, top]")
+    return T, D, E, F, experts.shape[1]
+
+
+def moe_experts_plain(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, experts: torch.Tensor,
+                      weights: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """float32 [T, D]: sum over a token's experts of down_e(act(gate_up_e (w h))), by the plain kernels."""
+    _gpu(h, gate_up, down, experts, weights)
+    T, D, E, F, top = _check_experts(h, gate_up, down, experts, weights, "moe_experts_plain")
+    y = torch.empty(T * top, F, dtype=h.dtype, device=h.device)
+    out = torch.empty(T, D, dtype=torch.float32, device=h.device)
+    lib = library.core()
+    _check(lib, lib.pico_moe_experts_plain(_ptr(h), h.stride(0) if T > 1 else D, _dt(h), _ptr(gate_up), _ptr(down),
+                                           _ptr(experts), _ptr(weights), _ptr(y), _ptr(out), T, top, E, F, D,
+                                           c_float(limit), c_float(alpha), _stream()))
     return out

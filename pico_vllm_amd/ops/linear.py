@@ -117,6 +117,13 @@ class Linear:
             return kernels.gemm_skinny(x, self.weight, None, kernels.EPI_SWIGLU)
         return kernels.swiglu(self(x))
 
+    def relu2(self, x: torch.Tensor) -> torch.Tensor:
+        """max(x W^T, 0)^2; with few rows the activation is the epilogue of the weight-streaming kernel."""
+        if self.weight.dtype == torch.bfloat16 and self.bias is None and kernels.skinny_ok(x, self.weight):
+            return kernels.gemm_skinny(x, self.weight, None, kernels.EPI_RELU2)
+        y = self(x)
+        return kernels.relu2(y, out=y)
+
     def partial(self, x: torch.Tensor) -> torch.Tensor:
         """x W^T as something a norm's ``add_norm`` takes as delta: [T, N], or, when the matrix is
         too small to fill the chip with one workgroup per output tile, a float32 stack [S, T, N] of

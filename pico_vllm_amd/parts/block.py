@@ -1,6 +1,7 @@
 """Arrangements of parts into a layer."""
 from __future__ import annotations
 
+from ..ops import kernels
 from .base import Block, DeferredNorm
 from .registry import register_part
 
@@ -40,3 +41,23 @@ class PreNormBlock(Block):
         h = self._normed(p["norm2"], p["ff"], resid, a)
         f = p["ff"].forward(h, ctx)
         return self._after(h, resid), f
+
+
+@register_part("block", "parallel")
+class ParallelBlock(Block):
+    """h = norm1(x); x += mixer(h) + ff(h): one norm, and both sublayers read its output.  A layer without a
+    feed-forward names the part "none" in that slot.  The sums are float32: the mixer's output joins the residual stream
+    at once, the feed-forward's is handed on as ``pending`` and the next norm adds it."""
+    slot_categories = {"norm1": "norm", "mixer": "mixer", "ff": "feed_forward"}
+    graph_safe_prompts = True
+
+    def forward(self, resid, pending, ctx, cache):
+        p = self.parts
+        h = p["norm1"].add_norm(resid, pending)
+        a = p["mixer"].forward(h, ctx, cache)
+        f = p["ff"].forward(h, ctx)
+        if f is None:
+            return resid, a
+        for delta in (a if a.dim() == 3 else (a,)):            # a stack of partial sums: each in turn
+            kernels.residual_add(resid, delta)
+        return resid, f

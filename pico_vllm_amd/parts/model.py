@@ -9,12 +9,18 @@ from ..config.registry import load_model_description
 from ..ops import kernels
 from ..ops.linear import Linear
 from ..weights.loader import load_checkpoint
-from . import attention, block, mlp, norm, rotary  # noqa: F401  (register the parts)
+from . import attention, attention_bias, block, mlp, moe, norm, positions, rotary  # noqa: F401  (register the parts)
 from .base import Block, StepContext
 from .registry import build_part, part_class
 from .spec import CacheSpec, ModelSpec, ParamSpec
 
 _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def tensor_name(*pieces: str) -> str:
+    """A checkpoint name from its pieces (layer prefix, part prefix, the part's own name); empty pieces are left
+    out, so a part whose prefix is the tensor's whole name declares the name ""."""
+    return ".".join(p for p in pieces if p)
 
 
 def _build_layer(lspec, act_dtype) -> Tuple[Block, Dict[str, str]]:
@@ -35,7 +41,7 @@ def _layer_params(lspec, blk: Block, sub: Dict[str, str]) -> List[Tuple[str, str
     out = []
     for slot, part in blk.parts.items():
         for p in part.param_specs():
-            full = f"{lspec.prefix}.{sub[slot]}.{p.name}"
+            full = tensor_name(lspec.prefix, sub[slot], p.name)
             out.append((slot, full, ParamSpec(full, p.shape, p.role, p.std)))
     return out
 
@@ -48,9 +54,9 @@ def model_param_specs(spec: ModelSpec) -> List[ParamSpec]:
         out += [p for _, _, p in _layer_params(lspec, blk, sub)]
     for prefix, pspec in tuple(spec.before_layers) + tuple(spec.after_layers):
         part = build_part("stream", pspec, act_dtype=torch.float32)
-        out += [ParamSpec(f"{prefix}.{p.name}" if prefix else p.name, p.shape, p.role, p.std) for p in part.param_specs()]
+        out += [ParamSpec(tensor_name(prefix, p.name), p.shape, p.role, p.std) for p in part.param_specs()]
     fn = build_part("norm", spec.final_norm, act_dtype=torch.float32)
-    out += [ParamSpec(f"{spec.final_norm_name}.{p.name}", p.shape, p.role, p.std) for p in fn.param_specs()]
+    out += [ParamSpec(tensor_name(spec.final_norm_name, p.name), p.shape, p.role, p.std) for p in fn.param_specs()]
     if spec.head_name:
         out.append(ParamSpec(spec.head_name, (spec.vocab_size, spec.hidden_size)))
     if spec.head_bias_name:
@@ -102,13 +108,12 @@ class DecoderModel:
         self.embed = tensors[spec.embed_name].to(dev).contiguous()
         for lspec, blk, sub in zip(spec.layers, self.layers, self._sub):
             for slot, part in blk.parts.items():
-                pre = f"{lspec.prefix}.{sub[slot]}."
-                part.load({p.name: tensors[pre + p.name] for p in part.param_specs()}, dev, self.dtype)
+                part.load({p.name: tensors[tensor_name(lspec.prefix, sub[slot], p.name)] for p in part.param_specs()},
+                          dev, self.dtype)
         for prefix, part in self.before + self.after:
-            pre = prefix + "." if prefix else ""
-            part.load({p.name: tensors[pre + p.name] for p in part.param_specs()}, dev, self.dtype)
-        pre = spec.final_norm_name + "."
-        self.final_norm.load({p.name: tensors[pre + p.name] for p in self.final_norm.param_specs()}, dev, self.dtype)
+            part.load({p.name: tensors[tensor_name(prefix, p.name)] for p in part.param_specs()}, dev, self.dtype)
+        self.final_norm.load({p.name: tensors[tensor_name(spec.final_norm_name, p.name)]
+                              for p in self.final_norm.param_specs()}, dev, self.dtype)
         self.head = Linear(tensors[spec.head_name].to(dev) if spec.head_name else self.embed,
                            tensors[spec.head_bias_name].to(dev) if spec.head_bias_name else None)
 

@@ -16,15 +16,16 @@ class RMSNorm(Norm):
     """y = x / sqrt(mean(x^2) + eps) * weight, in float32 (pico_vllm/RMSNorm.py:22-31)."""
     graph_safe_prompts = True
 
-    def __init__(self, size: int, eps: float, act_dtype: torch.dtype = torch.bfloat16):
-        self.size, self.eps, self.act_dtype = size, eps, act_dtype
+    def __init__(self, size: int, eps: float, act_dtype: torch.dtype = torch.bfloat16, weight_name: str = "weight"):
+        # weight_name: the gain's name behind the part's prefix; "" where the prefix itself names the tensor
+        self.size, self.eps, self.act_dtype, self.weight_name = size, eps, act_dtype, weight_name
         self.weight: Optional[torch.Tensor] = None
 
     def param_specs(self) -> List[ParamSpec]:
-        return [ParamSpec("weight", (self.size,), role="norm")]
+        return [ParamSpec(self.weight_name, (self.size,), role="norm")]
 
     def load(self, tensors: Dict[str, torch.Tensor], device, dtype) -> None:
-        self.weight = tensors["weight"].to(device=device, dtype=torch.float32).contiguous()
+        self.weight = tensors[self.weight_name].to(device=device, dtype=torch.float32).contiguous()
 
     def add_norm(self, resid, delta, rows=None):
         return kernels.add_rmsnorm(resid, delta, self.weight, self.eps, self.act_dtype, rows)
