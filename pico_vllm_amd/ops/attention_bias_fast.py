@@ -1,9 +1,79 @@
-"""The matrix-core kernels of the attention with a distance penalty, and the choice between them."""
+"""The matrix-core kernel of the attention with a distance penalty, and when it serves."""
 from __future__ import annotations
 
+import ctypes
 from typing import Optional
 
+import torch
 
-def choose(mixer) -> Optional[object]:
-    """The matrix-core kernels for this mixer's sizes, or None where the plain kernel serves."""
-    return None
+from . import library
+from .attention_fast import compute_units
+from .kernels import KernelError, _check, _check_cache2, _ptr, _stream
+
+c_float = ctypes.c_float
+
+
+def supported(key_dim: int, value_dim: int) -> bool:
+    """Key sizes in steps of 32 up to 512 and value sizes in steps of 16 up to 256; anything else goes to the plain kernel."""
+    return key_dim % 32 == 0 and 32 <= key_dim <= 512 and value_dim % 16 == 0 and 16 <= value_dim <= 256
+
+
+class FastBiasAttention:
+    def __init__(self, nq: int, nkv: int, key_dim: int, value_dim: int, scale: float, window: int = 0,
+                 temp_coef: float = 0.0, temp_every: int = 0, slope_span: float = 0.0):
+        self.nq, self.nkv, self.dk, self.dv = nq, nkv, key_dim, value_dim
+        self.scale, self.window, self.temp_coef, self.temp_every, self.slope_span = scale, window, temp_coef, temp_every, slope_span
+        self.lib = library.attention_bias_library(key_dim, value_dim)
+        if self.lib.pico_attnb_key_dim() != key_dim or self.lib.pico_attnb_value_dim() != value_dim:
+            raise KernelError("attention library was built for other sizes")
+        self.cus = compute_units()
+
+    def split(self, num_tokens: int) -> bool:
+        """Whether the four waves of a workgroup share ONE block of 16 query columns (few blocks: the chip is filled
+        by cutting their keys) or take a block each.  Decided from the number of tokens of the step alone."""
+        R = self.nq // self.nkv
+        blocks = -(-num_tokens // max(1, 16 // R)) * -(-R // 16) * self.nkv
+        return blocks < 8 * self.cus
+
+    def plan(self, ctx) -> tuple:
+        return (bool(self.split(ctx.num_tokens)),)
+
+    def run(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, positions, num_seqs: int,
+            split: Optional[bool] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """q [T, >= nq * dk] bfloat16 (row stride free); any mixture of portions and single tokens; returns [T, nq * dv]."""
+        T = q.shape[0]
+        pages, P = _check_cache2(k_cache, v_cache, self.nkv, self.dk, self.dv)
+        if not q.is_cuda or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
+            raise KernelError("matrix-core attention wants bfloat16 tensors on the GPU")
+        if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < self.nq * self.dk or (T > 1 and q.stride(0) % 8) or q.data_ptr() % 16:
+            raise KernelError("q must be [T, >= nq*dk] with unit stride along the row and 16-byte aligned rows")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous() \
+                or block_table.shape[0] < num_seqs:
+            raise KernelError("block_table must be contiguous int32 [sequences, pages]")
+        for t, n in ((cu_seqlens, num_seqs + 1), (positions, T)):
+            if t.dtype != torch.int32 or t.numel() < n or not t.is_contiguous():
+                raise KernelError("sequence metadata must be contiguous int32")
+        if P < 8 or P & (P - 1):
+            raise KernelError("matrix-core attention wants pages of a power of two of at least 8 tokens")
+        if out is None:
+            out = torch.empty(T, self.nq * self.dv, dtype=torch.bfloat16, device=q.device)
+        if split is None:
+            split = self.split(T)
+        _check(self.lib, self.lib.pico_attnb(
+            _ptr(q), q.stride(0) if T > 1 else q.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+            _ptr(cu_seqlens), _ptr(positions), num_seqs, T, _ptr(out), self.nq, self.nkv, self.dk, self.dv, P, pages,
+            c_float(self.scale), self.window, c_float(self.temp_coef), self.temp_every, c_float(self.slope_span),
+            1 if split else 0, _stream()))
+        return out
+
+    def __call__(self, qkv, cache, block_table, ctx):
+        return self.run(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.positions, ctx.num_seqs,
+                        split=self.plan(ctx)[0])
+
+
+def choose(mixer) -> Optional[FastBiasAttention]:
+    """The matrix-core kernel for this mixer's sizes, or None where the plain kernel serves."""
+    if not supported(mixer.dk, mixer.dv):
+        return None
+    return FastBiasAttention(mixer.nq, mixer.nkv, mixer.dk, mixer.dv, mixer.scale, mixer.window, mixer.temp_coef,
+                             mixer.temp_every, mixer.slope_span)

@@ -32,6 +32,8 @@ CORE_SOURCES = ("errors.hip", "elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip"
 
 ATTN_SOURCES = ("errors.hip", "attention_mfma.hip")
 
+ATTN_BIAS_SOURCES = ("errors.hip", "attention_bias_mfma.hip")
+
 PEAK_SOURCES = ("errors.hip", "peaks.hip")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
@@ -142,15 +144,24 @@ def attention_library(head_dim: int) -> ctypes.CDLL:
     return load_library(f"pico_attn_d{head_dim}", ATTN_SOURCES, (f"-DPICO_HEAD_DIM={head_dim}",))
 
 
+def attention_bias_library(key_dim: int, value_dim: int) -> ctypes.CDLL:
+    """The matrix-core kernel of the attention with a distance penalty, specialised for one pair of sizes."""
+    return load_library(f"pico_attnb_k{key_dim}_v{value_dim}", ATTN_BIAS_SOURCES,
+                        (f"-DPICO_DK={key_dim}", f"-DPICO_DV={value_dim}"))
+
+
 def peaks() -> ctypes.CDLL:
     """The two measuring kernels of the benchmark (a read stream, a matrix-core loop)."""
     return load_library("pico_peaks", PEAK_SOURCES)
 
 
-def build_all(head_dims: Iterable[int] = tuple(range(16, 257, 16)), force: bool = True) -> List[str]:
+def build_all(head_dims: Iterable[int] = tuple(range(16, 257, 16)), force: bool = True,
+              bias_dims: Iterable[tuple] = ((64, 32), (64, 64), (128, 64), (128, 128))) -> List[str]:
     """Compile everything (used by the build check); returns the paths."""
     out = [build_library("pico_core", CORE_SOURCES, force=force), build_library("pico_peaks", PEAK_SOURCES, force=force)]
     if os.path.isfile(os.path.join(CSRC, "attention_mfma.hip")):
         for d in head_dims:
             out.append(build_library(f"pico_attn_d{d}", ATTN_SOURCES, (f"-DPICO_HEAD_DIM={d}",), force=force))
+    for dk, dv in bias_dims:
+        out.append(build_library(f"pico_attnb_k{dk}_v{dv}", ATTN_BIAS_SOURCES, (f"-DPICO_DK={dk}", f"-DPICO_DV={dv}"), force=force))
     return out

@@ -115,6 +115,16 @@ def route(h: torch.Tensor, router: torch.Tensor, top: int):
     return experts, weights
 
 
+def router_margins(h: torch.Tensor, router: torch.Tensor, top: int) -> torch.Tensor:
+    """How far every token's choice is from being another: the gap between its last chosen and its first rejected
+    router logit, in units of the logits' spread (infinite where every expert is chosen)."""
+    z = h @ router.T
+    if top >= z.shape[-1]:
+        return torch.full((h.shape[0],), float("inf"), dtype=h.dtype)
+    s, _ = torch.sort(z, -1, descending=True)
+    return (s[:, top - 1] - s[:, top]) / z.std()
+
+
 def moe_ff(h: torch.Tensor, w: Dict[str, torch.Tensor], mlp: dict) -> torch.Tensor:
     """Sum over a token's chosen experts of expert(weight * h)."""
     experts, weights = route(h, w["router"], mlp["router"]["top"])
@@ -130,8 +140,9 @@ def _sub(tensors: Dict[str, torch.Tensor], prefix: str, dtype) -> Dict[str, torc
 
 
 def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.float64, layers_out: Optional[List] = None,
-            fast: bool = True) -> torch.Tensor:
-    """Logits [n, vocab] of one whole sequence.  ``layers_out``: a list that receives the residual stream after every layer."""
+            fast: bool = True, margins_out: Optional[List] = None) -> torch.Tensor:
+    """Logits [n, vocab] of one whole sequence.  ``layers_out``: a list that receives the residual stream after every
+    layer; ``margins_out``: one that receives ``router_margins`` of every routed layer."""
     eps = config["norm"]["eps"]
     x = embed_tokens(tokens, tensors["embed"].to(dtype), tensors["pos"].to(dtype))
     v_first = None
@@ -147,6 +158,8 @@ def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.
         mlp = layer.get("mlp")
         if mlp:
             w = _sub(tensors, f"l{i}.mlp.", dtype)
+            if mlp["kind"] == "moe" and margins_out is not None:
+                margins_out.append(router_margins(h, w["router"], mlp["router"]["top"]))
             delta = delta + (dense_ff(h, w) if mlp["kind"] == "dense" else moe_ff(h, w, mlp))
         x = x + delta
         if layers_out is not None:
