@@ -668,3 +668,51 @@ def moe_experts_plain(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor
                                            _ptr(experts), _ptr(weights), _ptr(y), _ptr(out), T, top, E, F, D,
                                            c_float(limit), c_float(alpha), _stream()))
     return out
+
+
+MOE_STREAM_ROWS = 32        # up to this many (token, expert) rows every row streams its expert's matrices
+
+
+def moe_fast_ok(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor) -> bool:
+    """Whether the bfloat16 kernels take these operands (sizes in multiples of 8, 16-byte aligned rows)."""
+    return (h.dtype == torch.bfloat16 and gate_up.dtype == torch.bfloat16 and down.dtype == torch.bfloat16
+            and h.dim() == 2 and h.stride(1) == 1 and h.shape[1] % 8 == 0 and down.shape[2] % 8 == 0
+            and (h.stride(0) % 8 == 0 or h.shape[0] == 1) and h.data_ptr() % 16 == 0
+            and gate_up.data_ptr() % 16 == 0 and down.data_ptr() % 16 == 0 and gate_up.shape[0] <= 1024)
+
+
+def moe_grouped_rows(tokens: int, top: int) -> bool:
+    """Whether a step of this many tokens sorts its rows by expert and multiplies on the matrix cores (decided from
+    the step's size alone)."""
+    return tokens * top > MOE_STREAM_ROWS
+
+
+def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, experts: torch.Tensor,
+                weights: torch.Tensor, limit: float, alpha: float, grouped: Optional[bool] = None) -> torch.Tensor:
+    """The experts' outputs in bfloat16 storage: float32 [T, D] (few rows: each streams its expert's matrices), or a
+    float32 stack [top, T, D] whose sum over the first index it is (many rows: sorted by expert on the device and
+    multiplied on the matrix cores)."""
+    _gpu(h, gate_up, down, experts, weights)
+    T, D, E, F, top = _check_experts(h, gate_up, down, experts, weights, "moe_experts")
+    if not moe_fast_ok(h, gate_up, down):
+        raise KernelError("moe_experts: bfloat16 operands with sizes in multiples of 8 and 16-byte aligned rows")
+    lib = library.core()
+    ldh = h.stride(0) if T > 1 else D
+    if grouped is None:
+        grouped = moe_grouped_rows(T, top)
+    if not grouped:
+        y = torch.empty(T * top, F, dtype=h.dtype, device=h.device)
+        out = torch.empty(T, D, dtype=torch.float32, device=h.device)
+        _check(lib, lib.pico_moe_experts_rows(_ptr(h), ldh, _ptr(gate_up), _ptr(down), _ptr(experts), _ptr(weights),
+                                              _ptr(y), _ptr(out), T, top, E, F, D, c_float(limit), c_float(alpha), _stream()))
+        return out
+    bm = lib.pico_moe_tile_rows()
+    tiles = (T * top + E * (bm - 1)) // bm
+    sorted_rows = torch.empty(tiles * bm, dtype=torch.int32, device=h.device)
+    tile_expert = torch.empty(tiles, dtype=torch.int32, device=h.device)
+    y = torch.empty(tiles * bm, F, dtype=h.dtype, device=h.device)
+    out = torch.empty(top, T, D, dtype=torch.float32, device=h.device)
+    _check(lib, lib.pico_moe_experts_grouped(_ptr(h), ldh, _ptr(gate_up), _ptr(down), _ptr(experts), _ptr(weights),
+                                             _ptr(sorted_rows), _ptr(tile_expert), tiles, _ptr(y), _ptr(out), T, top, E, F,
+                                             D, c_float(limit), c_float(alpha), _stream()))
+    return out[0] if top == 1 else out

@@ -77,4 +77,11 @@ class RoutedExperts(FeedForward):
         down = self.down.weight.view(E, D, F)
         if x.dtype != gate_up.dtype:
             x = x.to(gate_up.dtype)
+        if kernels.moe_fast_ok(x, gate_up, down):
+            # few rows stream their experts' matrices; many are sorted by expert and go to the matrix cores.  The
+            # second gives one float32 slab a slot: the next norm adds them up
+            return kernels.moe_experts(x, gate_up, down, experts, weights, self.limit, self.act_alpha)
         return kernels.moe_experts_plain(x, gate_up, down, experts, weights, self.limit, self.act_alpha)
+
+    def graph_variant(self, ctx: StepContext) -> tuple:
+        return (("routed_experts", kernels.moe_grouped_rows(ctx.num_tokens, self.top)),)

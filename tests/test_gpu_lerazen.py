@@ -297,11 +297,43 @@ def test_routed_experts(sizes, dtype):
     w = {n: t.to(torch.bfloat16) for n, t in w.items()}
     part.load(w, DEV, dtype)
     x = torch.randn(T, D).to(dtype)
-    got = part.forward(x.to(DEV), None).float().cpu()
+    got = part.forward(x.to(DEV), None)
+    got = (got.sum(0) if got.dim() == 3 else got).float().cpu()          # one slab a slot where the rows were sorted
     want = P.moe_ff(x.double(), {n: t.double() for n, t in w.items()},
                     {"router": {"experts": E, "top": top}, "expert": {"ff": F, "limit": 0.8}})
     tol = 2e-5 if dtype == torch.float32 else 3e-2
     assert torch.allclose(got.double(), want, atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("grouped", [False, True])
+@pytest.mark.parametrize("sizes", [(1, 6, 1, 8, 8), (3, 4, 2, 72, 40), (20, 3, 3, 104, 136), (500, 8, 2, 192, 256),
+                                   (130, 40, 1, 64, 64)])
+def test_expert_kernels_agree(sizes, grouped):
+    """Both bfloat16 paths (rows that stream their expert's matrices; rows sorted by expert for the matrix cores) against
+    the plain kernel, with experts that get no row, one row, and more rows than a tile holds."""
+    from pico_vllm_amd.ops import kernels
+    T, E, top, F, D = sizes
+    g = torch.Generator().manual_seed(T + E)
+    h = torch.randn(T, D, generator=g).bfloat16().to(DEV)
+    gate_up = (torch.randn(E, 2 * F, D, generator=g) * D ** -0.5).bfloat16().to(DEV)
+    down = (torch.randn(E, D, F, generator=g) * F ** -0.5).bfloat16().to(DEV)
+    z = torch.randn(T, E, generator=g) * 2
+    z[:, 0] -= 50                                                        # nobody chooses the first expert ...
+    if E > 4:
+        z[: T // 2, 1] += 50                                             # ... and half of the tokens the second
+        z[T // 2, 2] += 60
+    experts, weights = kernels.moe_route(z.to(DEV), top)
+    want = kernels.moe_experts_plain(h, gate_up, down, experts, weights, 0.9, 1.702)
+    got = kernels.moe_experts(h, gate_up, down, experts, weights, 0.9, 1.702, grouped=grouped)
+    got = got.sum(0) if got.dim() == 3 else got
+    assert got.shape == want.shape
+    assert float((got - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max()))
+    # the same rows among others give the same bits: a row's result does not depend on its company
+    few = slice(0, max(1, T // 3))
+    again = kernels.moe_experts(h[few].contiguous(), gate_up, down, experts[few].contiguous(), weights[few].contiguous(),
+                                0.9, 1.702, grouped=grouped)
+    again = again.sum(0) if again.dim() == 3 else again
+    assert torch.equal(again, got[few])
 
 
 def test_route_picks_the_largest_scores():
