@@ -7,6 +7,9 @@
                                                             (64 requests, prompts of 128..4096 tokens, 256 new tokens each,
                                                              continuous batching with prompts cut into portions)
 
+  python bench.py --workload designs --layers 4             (Lerazen beside the Qwen2.5 shape of equal size, at two sizes:
+                                                             decode at batch 1 and 8, the 2,048-token prefill)
+
   python bench.py --workload long --shape 32b --device-weights --context 32768
                                                             (one 16k-token prompt in portions of 2,048, then decode at
                                                              batch 1 and 8 with contexts ending at the context length;
@@ -47,7 +50,11 @@ from pico_vllm_amd.config.presets import preset   # noqa: E402  (needs ROOT on t
 # name -> (what the record calls it, the configuration as its config.json would hold it); the default run is the
 # Qwen2.5-1.5B shape, the others are measured with fewer layers when asked (--layers)
 SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", preset("1.5b")), "7b": ("Qwen2.5-7B shape", preset("7b")),
-          "32b": ("Qwen2.5-32B shape", preset("32b"))}
+          "32b": ("Qwen2.5-32B shape", preset("32b")),
+          "lerazen-1.5b": ("Lerazen at the 1.5B shape's sizes", preset("lerazen-1.5b")),
+          "lerazen-7b": ("Lerazen at the 7B shape's sizes", preset("lerazen-7b"))}
+# --workload designs: (a design's configuration, the closest existing model at equal size)
+DESIGN_PAIRS = (("lerazen-1.5b", "1.5b"), ("lerazen-7b", "7b"))
 CONFIG = SHAPES["1.5b"][1]   # the shape being measured (set in main)
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
@@ -400,6 +407,38 @@ def other_shape_points(dtype, steps, warmup):
             "prefill_tflops": round(pf["tflops"], 1), "prefill_frac": round(pf["frac"], 4)}
 
 
+def design_points(dtype, layers, steps, warmup, only=None):
+    """Every pair of DESIGN_PAIRS with ``layers`` layers each (weights drawn on the GPU): decode at batch 1 and 8 with
+    contexts ending at the context length and the 2,048-token prefill, with what a step reads and computes."""
+    import torch
+    rows = []
+    for pair in DESIGN_PAIRS:
+        for key in pair:
+            if only and key not in only:
+                continue
+            name, raw = SHAPES[key]
+            arch, typed, _ = describe(raw)
+            cut = arch.with_layers(raw, layers) if layers else raw
+            model = device_model(cut, dtype)
+            torch.cuda.synchronize()
+            row = {"model": name, "architecture": arch.name, "layers_run": arch.sizes(arch.config_from_dict(cut))["layers"],
+                   "hidden": arch.sizes(typed)["hidden"], "weight_gbytes_a_step": round(model.num_weight_bytes() / 1e9, 3)}
+            for b in (1, 8):
+                r, model = decode_point("", model, dtype, b, steps, warmup)
+                row[f"decode_b{b}_tok_s"] = round(r["tok_s"], 1)
+                row[f"decode_b{b}_ms_per_step"] = round(r["ms_median"], 4)
+                row[f"decode_b{b}_hbm_frac"] = round(r["gbps"] * 1e9 / HBM_PEAK, 4)
+                log(f"{name} decode batch {b}: {r['tok_s']:.0f} tok/s, {r['ms_median']:.3f} ms/step, {r['gbps'] / 1e3:.2f} TB/s")
+            pf = prefill_point("", model, dtype, reps=5)
+            row.update(prefill_tok_s=round(pf["value"], 1), prefill_ms=round(pf["ms"], 4), prefill_tflops=round(pf["tflops"], 1),
+                       prefill_frac=round(pf["frac"], 4))
+            log(f"{name} prefill: {pf['value']:.0f} tok/s, {pf['ms']:.2f} ms, {pf['tflops']:.0f} TFLOP/s")
+            rows.append(row)
+            del model
+            torch.cuda.empty_cache()
+    return rows
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -419,10 +458,11 @@ def main() -> int:
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (default: the 1.5B shape)")
     ap.add_argument("--layers", type=int, default=0, help="run only this many layers of the shape (0: all)")
     ap.add_argument("--context", type=int, default=4096, help="context length at which the decode steps end")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "sweep"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "sweep", "designs"],
                     help="decode: the contract's steady decode steps; serve: many requests of mixed lengths at once; "
                          "long: one prompt of --prompt tokens in portions, then decode at batch 1 and 8 at the context length; "
-                         "sweep: decode from context 16 to the context length, the time of a step by context")
+                         "sweep: decode from context 16 to the context length, the time of a step by context; "
+                         "designs: each newer design beside the closest existing model at equal size (--layers of each)")
     ap.add_argument("--prompt", type=int, default=16384, help="prompt tokens of the long workload")
     ap.add_argument("--device-weights", action="store_true",
                     help="draw the random weights on the GPU instead of writing and reading a model folder")
@@ -488,6 +528,13 @@ def main() -> int:
         print(json.dumps({"metric": "sampling call", "unit": "us", "value": r["top_p"], "greedy": r["greedy"],
                           "temperature": r["temperature"], "top_p": r["top_p"], "rows": rows, "vocab": r["vocab"],
                           "p": top_p}))
+        return 0
+    if a.workload == "designs":
+        rows = design_points(a.dtype, a.layers, min(a.steps, 100), min(a.warmup, 10))
+        print(json.dumps({"metric": f"designs side by side: decode tok/s at batch 1 and 8 (context {CONTEXT}), prefill of {PREFILL_TOKENS} tokens",
+                          "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
+                          "data": "synthetic: random weights N(0, 0.02) drawn on the GPU, uniform random token ids",
+                          "context": CONTEXT, "rows": rows}), flush=True)
         return 0
     if a.write_model:
         write_random_model(a.write_model, CONFIG, seed=0)
@@ -556,8 +603,8 @@ def main() -> int:
                 "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
                 "data": "synthetic: random weights N(0, 0.02)" + (" drawn on the GPU" if a.device_weights else "") + ", uniform random token ids",
                 "config": {"model": shape_name, "layers": layers_full, "layers_run": sizes["layers"],
-                           "hidden": sizes["hidden"], "q_heads": sizes["q_heads"],
-                           "kv_heads": sizes["kv_heads"], "intermediate": sizes["intermediate"],
+                           "hidden": sizes["hidden"], "q_heads": sizes.get("q_heads"),
+                           "kv_heads": sizes.get("kv_heads"), "intermediate": sizes.get("intermediate"),
                            "vocab": sizes["vocab"], "seq_len": CONTEXT, "prompt": a.prompt, "portion": PREFILL_TOKENS,
                            "page_size": 16, "weight_gbytes": round(model.num_weight_bytes() / 1e9, 1)},
                 "long_prompt": {k: (round(v, 2) if isinstance(v, float) else v) for k, v in lp.items()},
@@ -575,10 +622,10 @@ def main() -> int:
             "config": {"model": shape_name, "global_batch": a.batch, "seq_len": CONTEXT,
                        "parallelism": "single GPU", "layers": layers_full,
                        "layers_run": sizes["layers"], "hidden": sizes["hidden"],
-                       "q_heads": sizes["q_heads"], "kv_heads": sizes["kv_heads"],
-                       "head_dim": sizes["head_dim"],
-                       "intermediate": sizes["intermediate"], "vocab": sizes["vocab"],
-                       "tied": sizes["tied"],
+                       "q_heads": sizes.get("q_heads"), "kv_heads": sizes.get("kv_heads"),
+                       "head_dim": sizes.get("head_dim"),
+                       "intermediate": sizes.get("intermediate"), "vocab": sizes["vocab"],
+                       "tied": sizes.get("tied"),
                        "page_size": 16, "prompt_len": int(main_res["prompt_len"]),
                        "context_in_timed_steps": round(main_res["context"], 1)},
             "roofline": {"bound": "hbm", "achieved": round(main_res["gbps"], 1), "peak": HBM_PEAK / 1e9,

@@ -24,8 +24,36 @@ PRESETS: Dict[str, Dict] = {
 }
 
 
+def _lerazen(vocab, width, layers, heads, kv_heads, dim, dense_ff, experts, top, expert_ff, window=1024, every_global=4,
+             max_positions=40960) -> Dict:
+    """A Lerazen configuration of a real model's proportions: dense and routed feed-forwards in turn, windowed layers
+    with every ``every_global``-th one unwindowed, values mixed with the first layer's."""
+    def mixer(i):
+        m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "v_mix": True,
+             "q_temp": {"coef": 0.4, "every": 512}}
+        if (i + 1) % every_global:
+            m["mask"] = {"size": window}
+        return m
+    dense = {"kind": "dense", "ff": dense_ff}
+    routed = {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}
+    return {"architecture": "Lerazen", "vocab": vocab, "width": width, "max_positions": max_positions, "norm": {"eps": 1e-6},
+            "layers": [{"type": "attention", "mixer": mixer(i), "mlp": routed if i % 2 else dense} for i in range(layers)]}
+
+
+# Lerazen at the sizes of the Qwen2.5 shapes above: the same width, heads and layers; a token multiplies as many
+# feed-forward weights (two matrices of 1.5 x the intermediate size where it is dense; ``top`` experts of three
+# matrices where it is routed).  Kept apart from PRESETS, whose keys are one architecture's.
+DESIGN_PRESETS: Dict[str, Dict] = {
+    "lerazen-1.5b": _lerazen(151936, 1536, 28, 12, 2, 128, 13440, 16, 2, 4480),
+    "lerazen-7b": _lerazen(152064, 3584, 28, 28, 4, 128, 28416, 32, 4, 4736),
+}
+
+
 def preset(name: str) -> Dict:
-    try:
-        return dict(PRESETS[name.lower()])
-    except KeyError:
-        raise ValueError(f"unknown configuration {name!r}; known: {', '.join(sorted(PRESETS))}") from None
+    import copy
+    key = name.lower()
+    if key in PRESETS:
+        return dict(PRESETS[key])
+    if key in DESIGN_PRESETS:
+        return copy.deepcopy(DESIGN_PRESETS[key])
+    raise ValueError(f"unknown configuration {name!r}; known: {', '.join(sorted(PRESETS) + sorted(DESIGN_PRESETS))}")

@@ -16,11 +16,19 @@
 // ---------------------------------------------------------------------------
 #define MOE_MAX_TOP 16
 
+// the `top` largest of a row's E logits z (the lowest index among equal ones) and their sigmoids
+__device__ __forceinline__ void route_row(const float* z, int E, int top, int* __restrict__ experts,
+                                          float* __restrict__ weights);
+
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int T, int E, int top,
                                                        int* __restrict__ experts, float* __restrict__ weights) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
-  const float* z = logits + (size_t)t * E;
+  route_row(logits + (size_t)t * E, E, top, experts + (size_t)t * top, weights + (size_t)t * top);
+}
+
+__device__ __forceinline__ void route_row(const float* z, int E, int top, int* __restrict__ experts,
+                                          float* __restrict__ weights) {
   int chosen[MOE_MAX_TOP];
   for (int k = 0; k < top; k++) {
     int best = -1;
@@ -33,9 +41,87 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
       if (best < 0 || v > bz) { best = e; bz = v; }     // NaN never wins over a number; the first of equals stays
     }
     chosen[k] = best;
-    experts[(size_t)t * top + k] = best;
-    weights[(size_t)t * top + k] = 1.0f / (1.0f + expf(-bz));
+    experts[k] = best;
+    weights[k] = 1.0f / (1.0f + expf(-bz));
   }
+}
+
+// ---------------------------------------------------------------------------
+// Router logits z = x Wr^T in float32 (Wr float32 [E, D]; x float32 or bfloat16).  A wave makes one expert's logit of
+// ROUTER_TOKENS tokens: its lanes split k (four k a lane and turn where D is a multiple of 4, else one: a chain a lane,
+// then the wave's tree, an order that depends on D alone).  grid (ceil(T / ROUTER_TOKENS), ceil(E / 4)).
+// ---------------------------------------------------------------------------
+#define ROUTER_TOKENS 4
+
+template <typename T> __device__ __forceinline__ void load4_f32(const T* p, float* o);
+template <> __device__ __forceinline__ void load4_f32<float>(const float* p, float* o) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+template <> __device__ __forceinline__ void load4_f32<bf16_t>(const bf16_t* p, float* o) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+  o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void moe_logits_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ Wr,
+                                                         int Tn, int E, int D, float* __restrict__ z) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = blockIdx.x * ROUTER_TOKENS, e = blockIdx.y * 4 + wave;
+  if (e >= E) return;
+  const float* w = Wr + (size_t)e * D;
+  const T* xr[ROUTER_TOKENS];
+  float acc[ROUTER_TOKENS];
+#pragma unroll
+  for (int i = 0; i < ROUTER_TOKENS; i++) {
+    xr[i] = x + (size_t)min(t0 + i, Tn - 1) * ldx;
+    acc[i] = 0.f;
+  }
+  if (VEC) {
+#pragma unroll 2
+    for (int k = lane * 4; k < D; k += 256) {
+      float wv[4], xv[4];
+      load4_f32<float>(w + k, wv);
+#pragma unroll
+      for (int i = 0; i < ROUTER_TOKENS; i++) {
+        load4_f32<T>(xr[i] + k, xv);
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i] = fmaf(xv[j], wv[j], acc[i]);
+      }
+    }
+  } else {
+    for (int k = lane; k < D; k += 64) {
+      const float wv = w[k];
+#pragma unroll
+      for (int i = 0; i < ROUTER_TOKENS; i++) acc[i] = fmaf(load_f32(xr[i] + k), wv, acc[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < ROUTER_TOKENS; i++) {
+    const float s = wave_sum(acc[i]);
+    if (lane == 0 && t0 + i < Tn) z[(size_t)(t0 + i) * E + e] = s;
+  }
+}
+
+// router logits into z [T, E], then the choice: two launches
+extern "C" int pico_moe_router(const void* x, int ldx, int dtype, const float* Wr, int T, int E, int D, int top,
+                               float* z, int* experts, float* weights, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && E > 0 && D > 0 && ldx >= D && top > 0 && top <= E && top <= MOE_MAX_TOP,
+               "pico_moe_router: %d of %d experts per token is outside what the kernel takes (at most %d)", top, E, MOE_MAX_TOP);
+  PICO_REQUIRE(dtype == PICO_DTYPE_F32 || dtype == PICO_DTYPE_BF16, "pico_moe_router: unknown dtype %d", dtype);
+  if (T == 0) return 0;
+  const dim3 grid((T + ROUTER_TOKENS - 1) / ROUTER_TOKENS, (E + 3) / 4);
+  PICO_REQUIRE(grid.y <= 65535, "pico_moe_router: too many experts");
+  const size_t esz = dtype == PICO_DTYPE_F32 ? 4 : 2;
+  const bool vec = D % 4 == 0 && ldx % 4 == 0 && (uintptr_t)x % (4 * esz) == 0 && (uintptr_t)Wr % 16 == 0;
+#define LAUNCH(TT, V) moe_logits_kernel<TT, V><<<grid, 256, 0, stream>>>((const TT*)x, ldx, Wr, T, E, D, z)
+  if (dtype == PICO_DTYPE_F32) { if (vec) LAUNCH(float, true); else LAUNCH(float, false); }
+  else { if (vec) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
+#undef LAUNCH
+  moe_route_kernel<<<(T + 63) / 64, 64, 0, stream>>>(z, T, E, top, experts, weights);
+  PICO_LAUNCH_CHECK();
+  return 0;
 }
 
 extern "C" int pico_moe_route(const float* logits, int T, int E, int top, int* experts, float* weights,

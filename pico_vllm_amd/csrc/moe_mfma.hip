@@ -15,10 +15,10 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-#define MOE_BM 64          // rows of a tile
+#define MOE_BM 128         // rows of a tile
 #define MOE_BN 128         // matrix rows (output columns) of a tile
-#define MOE_BK 32          // k of one stage
-#define MOE_LD 40          // LDS row stride in bfloat16: 80 bytes, a multiple of 16 that spreads rows over the banks
+#define MOE_BK 64          // k of one stage
+#define MOE_LD 72          // LDS row stride in bfloat16: 144 bytes, a multiple of 16 that spreads rows over the banks
 
 __device__ __forceinline__ float moe_act(float g, float u, float limit, float alpha) {
   g = fminf(g, limit);
@@ -194,7 +194,9 @@ __global__ __launch_bounds__(MOE_SORT_THREADS) void moe_sort_kernel(const int* _
 }
 
 // ---------------------------------------------------------------------------
-// The grouped product.  grid (tiles_cap, ceil(N / BN)); 4 waves as 2 x 2; a wave makes 32 rows x 2 blocks of 32 columns.
+// The grouped product.  grid (tiles_cap, ceil(N / columns of a tile)); a tile is MOE_BM rows x MOE_BN matrix rows, staged
+// MOE_BK k at a time (the next stage travels in registers while this one is multiplied); 4 waves as 2 x 2, a wave makes
+// 64 rows x 2 blocks of 32 columns with four v_mfma_f32_32x32x16_bf16 a k step.
 // UP:   A = gathered, scaled rows of h (K = D); B rows = 64 gate rows f0.. and 64 up rows F + f0..; a wave holds gate and
 //       up of the same 32 columns and writes act(gate, up) to y[p, f] (bfloat16).
 // DOWN: A = y rows of the tile (K = F); B rows = 128 rows n0.. of down_e; float32 to out[slot][token][n].
@@ -205,101 +207,137 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
                                                           const int* __restrict__ tile_expert,
                                                           const float* __restrict__ weights, bf16_t* __restrict__ y,
                                                           float* __restrict__ out, int T, int top, int F, int D,
-                                                          float limit, float alpha) {
+                                                          float limit, float alpha, int ntile, int ncol) {
   __shared__ __attribute__((aligned(16))) bf16_t As[MOE_BM * MOE_LD];
   __shared__ __attribute__((aligned(16))) bf16_t Bs[MOE_BN * MOE_LD];
   __shared__ int rows[MOE_BM];
-  const int tile = blockIdx.x;
+  // Which tile and which columns.  Workgroups go to the chip's eight dies in turn, and every die has a second-level
+  // cache of its own.  Tiles are taken in pairs (neighbours in the sorted order: mostly one expert's); pair p belongs to
+  // die p % 8, and a die's consecutive workgroups are the two tiles of a pair at the same columns, then at the next
+  // columns: what runs together on a die shares its operands.  grid: 8 * ceil(pairs / 8) * 2 * ncol, one-dimensional.
+  const int die = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int pair = (idx / (2 * ncol)) * 8 + die, rest = idx % (2 * ncol);
+  const int tile = 2 * pair + (rest & 1), col = rest >> 1;
+  if (tile >= ntile) return;
   const int e = tile_expert[tile];
   if (e < 0) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int K = UP ? D : F;
-  const int N = UP ? F : D;                                   // output columns of the whole product
-  const int c0 = blockIdx.y * (UP ? MOE_BN / 2 : MOE_BN);     // first output column of this tile
+  const int c0 = col * (UP ? MOE_BN / 2 : MOE_BN);            // first output column of this tile
   if (tid < MOE_BM) rows[tid] = sorted[(size_t)tile * MOE_BM + tid];
 
-  // what this thread stages: 8 k of one A row and of two B rows
-  const int srow = tid >> 2, sk = (tid & 3) * 8;
-  const bf16_t* a_src;
-  float a_w = 1.f;
-  bool a_ok;
-  if (UP) {
-    const int r = sorted[(size_t)tile * MOE_BM + srow];
-    a_ok = r >= 0;
-    a_src = A + (size_t)(a_ok ? r / top : 0) * lda;
-    a_w = a_ok ? weights[r] : 0.f;
-  } else {
-    a_ok = true;                                              // y has a row for every place of every tile
-    a_src = A + ((size_t)tile * MOE_BM + srow) * lda;
+  // what this thread stages: 8 k of four A rows and of four B rows (rows srow, srow + 32, ...); rows that do not exist
+  // point at a row that does and are cleared after the load, so that every load is unconditional
+  const int srow = tid >> 3, sk = (tid & 7) * 8;
+  const size_t erows = UP ? (size_t)2 * F : (size_t)D;
+#define MOE_STAGE_ROW(i, A_SRC, A_W, A_OK, B_SRC, B_OK)                                   \
+  const bf16_t* A_SRC;                                                                    \
+  const bf16_t* B_SRC;                                                                    \
+  float A_W = 1.f;                                                                        \
+  bool A_OK = true, B_OK;                                                                 \
+  {                                                                                       \
+    const int m = srow + 32 * (i);                                                        \
+    if (UP) {                                                                             \
+      const int r = sorted[(size_t)tile * MOE_BM + m];                                    \
+      A_OK = r >= 0;                                                                      \
+      A_SRC = A + (size_t)(A_OK ? r / top : 0) * lda + sk;                                \
+      A_W = A_OK ? weights[r] : 0.f;                                                      \
+      const int f = c0 + (m & 63);                                                        \
+      B_OK = f < F;                                                                       \
+      B_SRC = W + ((size_t)e * erows + (B_OK ? (m >> 6) * F + f : 0)) * K + sk;           \
+    } else {                                                                              \
+      A_SRC = A + ((size_t)tile * MOE_BM + m) * lda + sk;                                 \
+      B_OK = c0 + m < D;                                                                  \
+      B_SRC = W + ((size_t)e * erows + (B_OK ? c0 + m : 0)) * K + sk;                     \
+    }                                                                                     \
   }
-  const bf16_t* b_src[2];
-  bool b_ok[2];
-#pragma unroll
-  for (int i = 0; i < 2; i++) {
-    int wrow;                                                 // the row of the expert's matrix
-    if (UP) {
-      const int f = c0 + srow;
-      b_ok[i] = f < F;
-      wrow = i * F + f;
-    } else {
-      const int n = c0 + i * 64 + srow;
-      b_ok[i] = n < D;
-      wrow = n;
-    }
-    const size_t erows = UP ? (size_t)2 * F : (size_t)D;
-    b_src[i] = W + ((size_t)e * erows + (b_ok[i] ? wrow : 0)) * K;
-  }
+  MOE_STAGE_ROW(0, a_src0, a_w0, a_ok0, b_src0, b_ok0)
+  MOE_STAGE_ROW(1, a_src1, a_w1, a_ok1, b_src1, b_ok1)
+  MOE_STAGE_ROW(2, a_src2, a_w2, a_ok2, b_src2, b_ok2)
+  MOE_STAGE_ROW(3, a_src3, a_w3, a_ok3, b_src3, b_ok3)
+#undef MOE_STAGE_ROW
 
-  f32x16 acc0, acc1;
+  f32x16 acc00, acc01, acc10, acc11;
 #pragma unroll
-  for (int r = 0; r < 16; r++) { acc0[r] = 0.f; acc1[r] = 0.f; }
+  for (int r = 0; r < 16; r++) { acc00[r] = 0.f; acc01[r] = 0.f; acc10[r] = 0.f; acc11[r] = 0.f; }
 
   const uint4 zero = make_uint4(0, 0, 0, 0);
-  uint4 ra, rb0, rb1;
-  auto fetch = [&](int k0) {
-    const int k = k0 + sk;
-    const bool k_ok = k < K;                                  // K is a multiple of 8: 8 k are in or out together
-    ra = (a_ok && k_ok) ? *reinterpret_cast<const uint4*>(a_src + k) : zero;
-    rb0 = (b_ok[0] && k_ok) ? *reinterpret_cast<const uint4*>(b_src[0] + k) : zero;
-    rb1 = (b_ok[1] && k_ok) ? *reinterpret_cast<const uint4*>(b_src[1] + k) : zero;
-  };
-  fetch(0);
-  const int a_off = (wm * 32 + (lane & 31)) * MOE_LD + (lane >> 5) * 8;
-  const int b_row0 = UP ? wn * 32 : wn * 64, b_row1 = UP ? 64 + wn * 32 : wn * 64 + 32;
-  const int b_off0 = (b_row0 + (lane & 31)) * MOE_LD + (lane >> 5) * 8;
-  const int b_off1 = (b_row1 + (lane & 31)) * MOE_LD + (lane >> 5) * 8;
+  uint4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
+  // K is a multiple of 8: the 8 k of a load are in or out together; a load beyond K reads k = 0 .. and is cleared
+#define MOE_FETCH(k0)                                                      \
+  {                                                                        \
+    const bool k_ok = (k0) + sk < K;                                       \
+    const int ko = k_ok ? (k0) : 0;                                        \
+    ra0 = *reinterpret_cast<const uint4*>(a_src0 + ko);                    \
+    ra1 = *reinterpret_cast<const uint4*>(a_src1 + ko);                    \
+    ra2 = *reinterpret_cast<const uint4*>(a_src2 + ko);                    \
+    ra3 = *reinterpret_cast<const uint4*>(a_src3 + ko);                    \
+    rb0 = *reinterpret_cast<const uint4*>(b_src0 + ko);                    \
+    rb1 = *reinterpret_cast<const uint4*>(b_src1 + ko);                    \
+    rb2 = *reinterpret_cast<const uint4*>(b_src2 + ko);                    \
+    rb3 = *reinterpret_cast<const uint4*>(b_src3 + ko);                    \
+    if (!(a_ok0 && k_ok)) ra0 = zero;                                      \
+    if (!(a_ok1 && k_ok)) ra1 = zero;                                      \
+    if (!(a_ok2 && k_ok)) ra2 = zero;                                      \
+    if (!(a_ok3 && k_ok)) ra3 = zero;                                      \
+    if (!(b_ok0 && k_ok)) rb0 = zero;                                      \
+    if (!(b_ok1 && k_ok)) rb1 = zero;                                      \
+    if (!(b_ok2 && k_ok)) rb2 = zero;                                      \
+    if (!(b_ok3 && k_ok)) rb3 = zero;                                      \
+  }
+  MOE_FETCH(0)
+  const int frag = (lane & 31) * MOE_LD + (lane >> 5) * 8;    // a lane's place in a block of 32 rows
+  const int a_off = wm * 64 * MOE_LD + frag;
+  const int b_off0 = (UP ? wn * 32 : wn * 64) * MOE_LD + frag;
+  const int b_off1 = (UP ? 64 + wn * 32 : wn * 64 + 32) * MOE_LD + frag;
   for (int k0 = 0; k0 < K; k0 += MOE_BK) {
     __syncthreads();                                          // the last stage has been read
-    *reinterpret_cast<uint4*>(As + srow * MOE_LD + sk) = UP ? scale8(ra, a_w) : ra;
-    *reinterpret_cast<uint4*>(Bs + srow * MOE_LD + sk) = rb0;
-    *reinterpret_cast<uint4*>(Bs + (64 + srow) * MOE_LD + sk) = rb1;
+    {
+      bf16_t* as = As + srow * MOE_LD + sk;
+      bf16_t* bs = Bs + srow * MOE_LD + sk;
+      *reinterpret_cast<uint4*>(as) = UP ? scale8(ra0, a_w0) : ra0;
+      *reinterpret_cast<uint4*>(as + 32 * MOE_LD) = UP ? scale8(ra1, a_w1) : ra1;
+      *reinterpret_cast<uint4*>(as + 64 * MOE_LD) = UP ? scale8(ra2, a_w2) : ra2;
+      *reinterpret_cast<uint4*>(as + 96 * MOE_LD) = UP ? scale8(ra3, a_w3) : ra3;
+      *reinterpret_cast<uint4*>(bs) = rb0;
+      *reinterpret_cast<uint4*>(bs + 32 * MOE_LD) = rb1;
+      *reinterpret_cast<uint4*>(bs + 64 * MOE_LD) = rb2;
+      *reinterpret_cast<uint4*>(bs + 96 * MOE_LD) = rb3;
+    }
     __syncthreads();
-    if (k0 + MOE_BK < K) fetch(k0 + MOE_BK);                  // the next stage travels while this one is multiplied
+    if (k0 + MOE_BK < K) MOE_FETCH(k0 + MOE_BK)               // the next stage travels while this one is multiplied
 #pragma unroll
     for (int ks = 0; ks < MOE_BK; ks += 16) {
-      const bf16x8 a = *reinterpret_cast<const bf16x8*>(As + a_off + ks);
+      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(As + a_off + ks);
+      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(As + a_off + 32 * MOE_LD + ks);
       const bf16x8 b0 = *reinterpret_cast<const bf16x8*>(Bs + b_off0 + ks);
       const bf16x8 b1 = *reinterpret_cast<const bf16x8*>(Bs + b_off1 + ks);
-      acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, acc1, 0, 0, 0);
+      acc00 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc00, 0, 0, 0);
+      acc01 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc01, 0, 0, 0);
+      acc10 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc10, 0, 0, 0);
+      acc11 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc11, 0, 0, 0);
     }
   }
+#undef MOE_FETCH
   // a lane holds column lane % 32 of its blocks and rows 8 (r / 4) + 4 (lane / 32) + r % 4
-#pragma unroll
-  for (int r = 0; r < 16; r++) {
-    const int m = wm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-    if (UP) {
-      const int f = c0 + wn * 32 + (lane & 31);
-      if (f < F) y[((size_t)tile * MOE_BM + m) * F + f] = f32_to_bf16(moe_act(acc0[r], acc1[r], limit, alpha));
-    } else {
-      const int row = rows[m];
-      if (row < 0) continue;
-      float* o = out + ((size_t)(row % top) * T + row / top) * D;
-      const int n = c0 + wn * 64 + (lane & 31);
-      if (n < D) o[n] = acc0[r];
-      if (n + 32 < D) o[n + 32] = acc1[r];
-    }
+#define MOE_WRITE(i, ACC0, ACC1)                                                                                     \
+  _Pragma("unroll") for (int r = 0; r < 16; r++) {                                                                   \
+    const int m = wm * 64 + 32 * (i) + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);                                     \
+    if (UP) {                                                                                                        \
+      const int f = c0 + wn * 32 + (lane & 31);                                                                      \
+      if (f < F) y[((size_t)tile * MOE_BM + m) * F + f] = f32_to_bf16(moe_act(ACC0[r], ACC1[r], limit, alpha));      \
+    } else {                                                                                                         \
+      const int row = rows[m];                                                                                       \
+      if (row < 0) continue;                                                                                         \
+      float* o = out + ((size_t)(row % top) * T + row / top) * D;                                                    \
+      const int n = c0 + wn * 64 + (lane & 31);                                                                      \
+      if (n < D) o[n] = ACC0[r];                                                                                     \
+      if (n + 32 < D) o[n + 32] = ACC1[r];                                                                           \
+    }                                                                                                                \
   }
+  MOE_WRITE(0, acc00, acc01)
+  MOE_WRITE(1, acc10, acc11)
+#undef MOE_WRITE
 }
 
 extern "C" int pico_moe_tile_rows() { return MOE_BM; }
@@ -318,13 +356,16 @@ extern "C" int pico_moe_experts_grouped(const void* h, int ldh, const void* gate
   PICO_REQUIRE(R < (1ll << 30), "pico_moe_experts_grouped: too many rows");
   const long long need = (R + (long long)E * (MOE_BM - 1)) / MOE_BM;
   PICO_REQUIRE(tiles_cap >= need, "pico_moe_experts_grouped: room for %d tiles, %lld may be needed", tiles_cap, need);
-  const dim3 g1(tiles_cap, (F + MOE_BN / 2 - 1) / (MOE_BN / 2)), g2(tiles_cap, (D + MOE_BN - 1) / MOE_BN);
-  PICO_REQUIRE(g1.y <= 65535 && g2.y <= 65535, "pico_moe_experts_grouped: sizes beyond the grid");
+  const long long ncol1 = (F + MOE_BN / 2 - 1) / (MOE_BN / 2), ncol2 = (D + MOE_BN - 1) / MOE_BN;
+  const long long slots = ((tiles_cap + 1) / 2 + 7) / 8 * 8 * 2;       // tiles in pairs, pairs in eights
+  PICO_REQUIRE(slots * ncol1 < (1ll << 31) && slots * ncol2 < (1ll << 31), "pico_moe_experts_grouped: sizes beyond the grid");
   moe_sort_kernel<<<E, MOE_SORT_THREADS, 0, stream>>>(experts, (int)R, E, tiles_cap, sorted, tile_expert);
-  moe_grouped_kernel<true><<<g1, 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)gate_up, sorted, tile_expert,
-                                                   weights, (bf16_t*)y, nullptr, T, top, F, D, limit, alpha);
-  moe_grouped_kernel<false><<<g2, 256, 0, stream>>>((const bf16_t*)y, F, (const bf16_t*)down, sorted, tile_expert,
-                                                    nullptr, nullptr, out, T, top, F, D, limit, alpha);
+  moe_grouped_kernel<true><<<(unsigned)(slots * ncol1), 256, 0, stream>>>(
+      (const bf16_t*)h, ldh, (const bf16_t*)gate_up, sorted, tile_expert, weights, (bf16_t*)y, nullptr, T, top, F, D, limit,
+      alpha, tiles_cap, (int)ncol1);
+  moe_grouped_kernel<false><<<(unsigned)(slots * ncol2), 256, 0, stream>>>(
+      (const bf16_t*)y, F, (const bf16_t*)down, sorted, tile_expert, nullptr, nullptr, out, T, top, F, D, limit, alpha,
+      tiles_cap, (int)ncol2);
   PICO_LAUNCH_CHECK();
   return 0;
 }

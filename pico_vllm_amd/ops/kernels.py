@@ -639,6 +639,27 @@ def moe_route(logits: torch.Tensor, top: int):
     return experts, weights
 
 
+def moe_router(x: torch.Tensor, w_router: torch.Tensor, top: int):
+    """Router and choice: z = x w_router^T in float32 (w_router float32 [E, D]; x float32 or bfloat16 with
+    unit stride along the row), then as ``moe_route``: (experts int32 [T, top], weights float32 [T, top])."""
+    _gpu(x, w_router)
+    T, D = x.shape
+    E = w_router.shape[0]
+    if w_router.dtype != torch.float32 or w_router.dim() != 2 or w_router.shape[1] != D or not w_router.is_contiguous():
+        raise KernelError(f"moe_router: the router matrix must be contiguous float32 [experts, {D}]")
+    if x.stride(1) != 1:
+        raise KernelError("moe_router: activations must have unit stride along the row")
+    if not 1 <= top <= min(E, MOE_MAX_TOP):
+        raise KernelError(f"moe_router: {top} of {E} experts per token (at most {MOE_MAX_TOP})")
+    z = torch.empty(T, E, dtype=torch.float32, device=x.device)
+    experts = torch.empty(T, top, dtype=torch.int32, device=x.device)
+    weights = torch.empty(T, top, dtype=torch.float32, device=x.device)
+    lib = library.core()
+    _check(lib, lib.pico_moe_router(_ptr(x), x.stride(0) if T > 1 else D, _dt(x), _ptr(w_router), T, E, D, top,
+                                    _ptr(z), _ptr(experts), _ptr(weights), _stream()))
+    return experts, weights
+
+
 def _check_experts(h, gate_up, down, experts, weights, who):
     T, D = h.shape
     if gate_up.dim() != 3 or down.dim() != 3 or gate_up.shape[1] % 2:

@@ -71,8 +71,7 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         E, F, D = self.num_experts, self.expert_size, self.hidden_size
-        z = self.router(x, out_dtype=torch.float32)
-        experts, weights = kernels.moe_route(z, self.top)
+        experts, weights = kernels.moe_router(x, self.router.weight, self.top)
         gate_up = self.gate_up.weight.view(E, 2 * F, D)
         down = self.down.weight.view(E, D, F)
         if x.dtype != gate_up.dtype:

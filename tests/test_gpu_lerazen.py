@@ -345,6 +345,26 @@ def test_route_picks_the_largest_scores():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(1, 3, 1, 8), (7, 5, 5, 100), (70, 40, 3, 72), (33, 130, 16, 1536)])
+def test_router(sizes, dtype):
+    """Logits in float32 from the activations as they are stored, the largest scores chosen, their sigmoids the weights."""
+    from pico_vllm_amd.ops import kernels
+    T, E, top, D = sizes
+    g = torch.Generator().manual_seed(E)
+    x = torch.randn(T, D, generator=g).to(dtype)
+    w = torch.randn(E, D, generator=g) * D ** -0.5
+    z = x.double() @ w.double().t()
+    experts, weights = kernels.moe_router(x.to(DEV), w.to(DEV), top)
+    experts, weights = experts.cpu().long(), weights.cpu().double()
+    got_z = torch.gather(z, 1, experts)
+    assert torch.allclose(weights, torch.sigmoid(got_z), atol=1e-5)
+    assert bool((got_z[:, 1:] <= got_z[:, :-1] + 1e-5).all())                       # in falling order
+    rest = z.clone().scatter_(1, experts, -1e9)
+    assert bool((rest.max(1).values <= got_z[:, -1] + 1e-5).all())                  # nothing left out is larger
+    assert all(len(set(r)) == top for r in experts.tolist())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows", [1, 5, 64, 300])
 def test_squared_relu_feed_forward(rows, dtype):
     from pico_vllm_amd.parts.mlp import Relu2MLP
