@@ -42,6 +42,11 @@ struct BiasArgs {
   bf16_t* out;                 // [T, nq * DV]
   int num_seqs, nq, nkv, P, num_pages, window, temp_every;
   float scale, temp_coef, slope_span;
+  // chunks > 1 (SPLIT only): workgroup z of a block takes the z-th piece of the block's keys and leaves its sums
+  // unnormalised in parts_o [chunks][columns][DV] and its (maximum, sum) in parts_ml [chunks][columns][2]
+  int chunks, ncols;
+  float* parts_o;
+  float* parts_ml;
 };
 
 template <bool SPLIT>
@@ -102,11 +107,18 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
 
   const int pshift = 31 - __clz(a.P);                   // page sizes are powers of two
   const int stride = SPLIT ? 128 : 32;
-  const int first = (lo & ~31) + (SPLIT ? 32 * wave : 0);
-  if (ntok > 0 && first < hi) {
+  int begin = lo & ~31, end = hi;
+  if (SPLIT && a.chunks > 1) {
+    // pieces of whole turns of the four waves (128 keys), so the tiles are those of the uncut loop
+    const int piece = ((hi - begin + a.chunks - 1) / a.chunks + 127) & ~127;
+    begin += (int)blockIdx.z * piece;
+    end = min(hi, begin + piece);
+  }
+  const int first = begin + (SPLIT ? 32 * wave : 0);
+  if (ntok > 0 && first < end) {
     const int last_key = hi - 1, last_group = last_key / 8 * 8;
     const int row_key = 8 * (col >> 2) + (col & 3);     // key of this lane's row in tile 0; tile 1: 4 more
-    for (int key0 = first; key0 < hi; key0 += stride) {
+    for (int key0 = first; key0 < end; key0 += stride) {
       uint4 kr[2][KS];
       uint4 vr[DT];
       // positions beyond the range are clamped to its last key (group of 8, which lies in one page as pages hold at
@@ -183,7 +195,7 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
       }
     }
   }
-  float a0 = 1.f, L = l;
+  float a0 = 1.f, L = l, M_all = m;
   if (SPLIT) {
     // merge the four waves; lane (col, kq) of wave 0 holds value dimensions 16 tt + 4 kq + r of column `col`
     if (wave > 0) {
@@ -199,6 +211,7 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
 #pragma unroll
     for (int w = 0; w < 3; w++) M = fmaxf(M, xml[w][0][col]);
     const float m_use = (M == -INFINITY) ? 0.f : M;
+    M_all = M;
     a0 = __expf(m - m_use);
     float aw[3];
     L = l * a0;
@@ -218,6 +231,14 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
       }
   }
   if (!col_ok) return;
+  if (SPLIT && a.chunks > 1) {
+    const size_t c = (size_t)blockIdx.z * a.ncols + (size_t)t * a.nq + head;
+    float* po = a.parts_o + c * DV + 4 * kq;
+#pragma unroll
+    for (int tt = 0; tt < DT; tt++) *reinterpret_cast<f32x4*>(po + 16 * tt) = o[tt];
+    if (kq == 0) { a.parts_ml[2 * c] = M_all; a.parts_ml[2 * c + 1] = L; }
+    return;
+  }
   const float inv = 1.0f / L;
   bf16_t* orow = a.out + ((size_t)t * a.nq + head) * DV + 4 * kq;
 #pragma unroll
@@ -229,17 +250,38 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
   }
 }
 
+// The pieces of a column's keys put together: out = sum_z o_z e^(m_z - M) / sum_z l_z e^(m_z - M), z in ascending order.
+__global__ __launch_bounds__(DV <= 64 ? 64 : DV <= 128 ? 128 : 256) void attn_bias_merge_kernel(
+    const float* __restrict__ parts_o, const float* __restrict__ parts_ml, int chunks, int ncols, bf16_t* __restrict__ out) {
+  const int c = blockIdx.x, d = threadIdx.x;
+  if (d >= DV) return;
+  float M = -INFINITY;
+  for (int z = 0; z < chunks; z++) M = fmaxf(M, parts_ml[2 * ((size_t)z * ncols + c)]);
+  float L = 0.f, acc = 0.f;
+  for (int z = 0; z < chunks; z++) {
+    const size_t i = (size_t)z * ncols + c;
+    const float mz = parts_ml[2 * i];
+    const float w = mz == -INFINITY ? 0.f : __expf(mz - M);
+    L += parts_ml[2 * i + 1] * w;
+    acc += parts_o[i * DV + d] * w;
+  }
+  out[(size_t)c * DV + d] = f32_to_bf16(acc / L);
+}
+
 // split != 0: one block of 16 columns a workgroup, its keys shared by the four waves; else four blocks a workgroup.
 extern "C" int pico_attnb(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_table,
                           int max_pages, const int* cu_seqlens, const int* positions, int num_seqs, int T, void* out,
                           int nq, int nkv, int dk, int dv, int P, int num_pages, float scale, int window, float temp_coef,
-                          int temp_every, float slope_span, int split, hipStream_t stream) {
+                          int temp_every, float slope_span, int split, int chunks, float* parts_o, float* parts_ml,
+                          hipStream_t stream) {
   PICO_REQUIRE(dk == DK && dv == DV, "pico_attnb: built for keys of %d and values of %d, asked for %d and %d", DK, DV, dk, dv);
   PICO_REQUIRE(T >= 0 && num_seqs > 0 && nq > 0 && nkv > 0 && nq % nkv == 0 && max_pages > 0 && num_pages > 0,
                "pico_attnb: bad sizes");
   PICO_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "pico_attnb: the page size must be a power of two of at least 8, got %d", P);
   PICO_REQUIRE(q_stride >= nq * DK && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0, "pico_attnb: query rows must be 16-byte aligned");
   PICO_REQUIRE(nkv <= 65535 && window >= 0 && temp_every >= 0 && slope_span >= 0.f, "pico_attnb: bad constants");
+  PICO_REQUIRE(chunks >= 1 && chunks <= 65535 && (chunks == 1 || (split && parts_o && parts_ml)),
+               "pico_attnb: pieces of the keys go with one block a workgroup and need room for the parts");
   if (T == 0) return 0;
   const int R = nq / nkv;
   const int tpb = R >= 16 ? 1 : 16 / R, hb = R > 16 ? (R + 15) / 16 : 1;
@@ -248,10 +290,13 @@ extern "C" int pico_attnb(const void* q, int q_stride, const void* k_cache, cons
   PICO_REQUIRE(tiles < (1ll << 30), "pico_attnb: too many blocks");
   BiasArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
              cu_seqlens, positions, (bf16_t*)out, num_seqs, nq, nkv, P, num_pages, window, temp_every, scale, temp_coef,
-             slope_span};
-  if (split)
-    attn_bias_kernel<true><<<dim3((unsigned)tiles, nkv), 256, 0, stream>>>(a);
-  else
+             slope_span, chunks, T * nq, parts_o, parts_ml};
+  if (split) {
+    attn_bias_kernel<true><<<dim3((unsigned)tiles, nkv, chunks), 256, 0, stream>>>(a);
+    if (chunks > 1)
+      attn_bias_merge_kernel<<<T * nq, DV <= 64 ? 64 : DV <= 128 ? 128 : 256, 0, stream>>>(parts_o, parts_ml, chunks, T * nq,
+                                                                                           (bf16_t*)out);
+  } else
     attn_bias_kernel<false><<<dim3((unsigned)((tiles + 3) / 4), nkv), 256, 0, stream>>>(a);
   PICO_LAUNCH_CHECK();
   return 0;

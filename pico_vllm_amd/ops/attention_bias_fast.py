@@ -11,6 +11,7 @@ from .attention_fast import compute_units
 from .kernels import KernelError, _check, _check_cache2, _ptr, _stream
 
 c_float = ctypes.c_float
+MAX_CHUNKS = 32
 
 
 def supported(key_dim: int, value_dim: int) -> bool:
@@ -35,11 +36,22 @@ class FastBiasAttention:
         blocks = -(-num_tokens // max(1, 16 // R)) * -(-R // 16) * self.nkv
         return blocks < 8 * self.cus
 
+    def chunks(self, num_tokens: int, num_seqs: int) -> int:
+        """Into how many pieces every block's keys are cut, each piece a workgroup of its own (their parts are put
+        together by a second launch): as many as bring the step to two workgroups a compute unit, at most MAX_CHUNKS.
+        Decided from the step's size alone; a piece is a whole number of 128 keys, found on the device from the block's
+        own range of keys."""
+        if not self.split(num_tokens):
+            return 1
+        R = self.nq // self.nkv
+        blocks = (-(-num_tokens // max(1, 16 // R)) + num_seqs) * -(-R // 16) * self.nkv
+        return max(1, min(MAX_CHUNKS, -(-2 * self.cus // blocks)))
+
     def plan(self, ctx) -> tuple:
-        return (bool(self.split(ctx.num_tokens)),)
+        return (bool(self.split(ctx.num_tokens)), self.chunks(ctx.num_tokens, ctx.num_seqs))
 
     def run(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, positions, num_seqs: int,
-            split: Optional[bool] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+            split: Optional[bool] = None, out: Optional[torch.Tensor] = None, chunks: Optional[int] = None) -> torch.Tensor:
         """q [T, >= nq * dk] bfloat16 (row stride free); any mixture of portions and single tokens; returns [T, nq * dv]."""
         T = q.shape[0]
         pages, P = _check_cache2(k_cache, v_cache, self.nkv, self.dk, self.dv)
@@ -59,16 +71,24 @@ class FastBiasAttention:
             out = torch.empty(T, self.nq * self.dv, dtype=torch.bfloat16, device=q.device)
         if split is None:
             split = self.split(T)
+        if chunks is None:
+            chunks = self.chunks(T, num_seqs) if split else 1
+        parts_o = parts_ml = None
+        if chunks > 1:
+            if not split:
+                raise KernelError("pieces of the keys go with one block a workgroup")
+            parts_o = torch.empty(chunks, T * self.nq, self.dv, dtype=torch.float32, device=q.device)
+            parts_ml = torch.empty(chunks, T * self.nq, 2, dtype=torch.float32, device=q.device)
         _check(self.lib, self.lib.pico_attnb(
             _ptr(q), q.stride(0) if T > 1 else q.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
             _ptr(cu_seqlens), _ptr(positions), num_seqs, T, _ptr(out), self.nq, self.nkv, self.dk, self.dv, P, pages,
             c_float(self.scale), self.window, c_float(self.temp_coef), self.temp_every, c_float(self.slope_span),
-            1 if split else 0, _stream()))
+            1 if split else 0, chunks, _ptr(parts_o), _ptr(parts_ml), _stream()))
         return out
 
     def __call__(self, qkv, cache, block_table, ctx):
         return self.run(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.positions, ctx.num_seqs,
-                        split=self.plan(ctx)[0])
+                        split=self.plan(ctx)[0], chunks=self.plan(ctx)[1])
 
 
 def choose(mixer) -> Optional[FastBiasAttention]:

@@ -166,6 +166,8 @@ ATTN_CASES = [
     (3, 1, 24, 40, 5, (0.5, 3), 8, 9, 11),
     (40, 2, 32, 16, 70, None, 16, 64, 3),           # more than 16 heads a group
     (5, 1, 64, 64, 33, None, 16, 31, 34),           # heads a group that do not divide 16
+    (4, 2, 64, 32, None, (0.3, 100), 16, 1500, 2),  # many keys: pieces of several turns of the waves
+    (4, 2, 64, 32, 700, None, 16, 1203, 1),
 ]
 
 
@@ -192,9 +194,10 @@ def test_attention_kernels(case, dtype):
     if dtype == torch.bfloat16 and attention_bias_fast.supported(dk, dv):
         fast = attention_bias_fast.FastBiasAttention(H, G, dk, dv, scale, window or 0, tc, te, 8.0)
         cu = torch.tensor([0, new], dtype=torch.int32, device=DEV)
-        for split in (True, False):
-            got = fast.run(qd, K, V, bt, cu, pos, 1, split=split)
-            assert torch.allclose(got.cpu().double().view(new, H, dv), want, atol=tol, rtol=tol), f"split={split}"
+        # four blocks a workgroup; one block a workgroup; one block's keys in pieces that are put together afterwards
+        for split, chunks in ((False, 1), (True, 1), (True, 2), (True, 3), (True, 32)):
+            got = fast.run(qd, K, V, bt, cu, pos, 1, split=split, chunks=chunks)
+            assert torch.allclose(got.cpu().double().view(new, H, dv), want, atol=tol, rtol=tol), f"split={split} chunks={chunks}"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
