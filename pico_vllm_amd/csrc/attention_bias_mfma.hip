@@ -250,20 +250,28 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
   }
 }
 
+#define MAX_PIECES 64
 // The pieces of a column's keys put together: out = sum_z o_z e^(m_z - M) / sum_z l_z e^(m_z - M), z in ascending order.
 __global__ __launch_bounds__(DV <= 64 ? 64 : DV <= 128 ? 128 : 256) void attn_bias_merge_kernel(
     const float* __restrict__ parts_o, const float* __restrict__ parts_ml, int chunks, int ncols, bf16_t* __restrict__ out) {
+  // the pieces' maxima and sums once into LDS (one load a thread, all in flight together), then every thread its sum
+  __shared__ float ms[MAX_PIECES], ws[MAX_PIECES];
   const int c = blockIdx.x, d = threadIdx.x;
+  for (int z = d; z < chunks; z += blockDim.x) {
+    const float2 ml = *reinterpret_cast<const float2*>(parts_ml + 2 * ((size_t)z * ncols + c));
+    ms[z] = ml.x;
+    ws[z] = ml.y;
+  }
+  __syncthreads();
   if (d >= DV) return;
   float M = -INFINITY;
-  for (int z = 0; z < chunks; z++) M = fmaxf(M, parts_ml[2 * ((size_t)z * ncols + c)]);
+  for (int z = 0; z < chunks; z++) M = fmaxf(M, ms[z]);
   float L = 0.f, acc = 0.f;
+#pragma unroll 8
   for (int z = 0; z < chunks; z++) {
-    const size_t i = (size_t)z * ncols + c;
-    const float mz = parts_ml[2 * i];
-    const float w = mz == -INFINITY ? 0.f : __expf(mz - M);
-    L += parts_ml[2 * i + 1] * w;
-    acc += parts_o[i * DV + d] * w;
+    const float w = ms[z] == -INFINITY ? 0.f : __expf(ms[z] - M);
+    L += ws[z] * w;
+    acc += parts_o[((size_t)z * ncols + c) * DV + d] * w;
   }
   out[(size_t)c * DV + d] = f32_to_bf16(acc / L);
 }
@@ -280,7 +288,7 @@ extern "C" int pico_attnb(const void* q, int q_stride, const void* k_cache, cons
   PICO_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "pico_attnb: the page size must be a power of two of at least 8, got %d", P);
   PICO_REQUIRE(q_stride >= nq * DK && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0, "pico_attnb: query rows must be 16-byte aligned");
   PICO_REQUIRE(nkv <= 65535 && window >= 0 && temp_every >= 0 && slope_span >= 0.f, "pico_attnb: bad constants");
-  PICO_REQUIRE(chunks >= 1 && chunks <= 65535 && (chunks == 1 || (split && parts_o && parts_ml)),
+  PICO_REQUIRE(chunks >= 1 && chunks <= MAX_PIECES && (chunks == 1 || (split && parts_o && parts_ml)),
                "pico_attnb: pieces of the keys go with one block a workgroup and need room for the parts");
   if (T == 0) return 0;
   const int R = nq / nkv;
