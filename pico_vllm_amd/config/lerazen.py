@@ -161,6 +161,8 @@ def lerazen_spec(cfg: LerazenConfig) -> ModelSpec:
         run_order=[RunEntry(i) for i in range(len(layers))],
         final_norm=norm, final_norm_name="final.norm", head_name="head", eos_token_id=cfg.eos_token_id,
         max_position=cfg.max_positions,
+        # a checkpoint may hold a mixing scalar for a layer that does not mix: it is not used
+        ignored_tensors=tuple(f"l{i}.mix.vmix" for i, l in enumerate(cfg.layers) if not l.mixer.v_mix),
         before_layers=(("", PartSpec("learned_positions", {"size": cfg.width, "max_positions": cfg.max_positions,
                                                            "name": "pos"})),),
     )

@@ -10,7 +10,7 @@ import torch
 
 import plain_lerazen as P
 from gpu_util import DEV
-from lerazen_configs import CONFIGS, model_dir, tensors_of
+from lerazen_configs import CONFIGS, attention, config, dense, model_dir, moe, tensors_of
 
 pytestmark = pytest.mark.gpu
 
@@ -492,6 +492,41 @@ def test_batch_equals_each_alone(dtype):
         elif not tainted(name, reqs[key[0]], key[1]):
             assert float(row_errors(a[key][None], b[key][None])[0]) <= BOUND[dtype]
     compare(name, dtype, a, reqs)
+
+
+def draw_config(seed):
+    """A configuration drawn at random: sizes, head counts, windows, constants and the order of layers all differ from
+    the hand-picked ones, and include the values that make mechanisms vanish (a window of 1, one expert, one head)."""
+    rng = random.Random(1000 + seed)
+    width = rng.choice([24, 40, 64, 72, 96, 128])
+    kv_heads, vdim = rng.choice([1, 2, 3]), rng.choice([8, 16, 24, 32, 48, 64])      # the same in all layers that mix values
+    layers = []
+    for _ in range(rng.randint(1, 5)):
+        per = rng.choice([1, 2, 4, 6])
+        dim = rng.choice([8, 16, 24, 32, 64, 96])
+        m = attention(kv_heads * per, kv_heads, dim, vdim, window=rng.choice([None, 1, 2, 7, 16, 17, 40, 100]),
+                      temp=rng.choice([None, (0.9, 1), (0.3, 7), (1.5, 64)]), v_mix=rng.random() < 0.7,
+                      scale=rng.choice([None, 0.31, 2.0 * dim ** -0.5]))
+        kind = rng.choice(["none", "dense", "moe", "moe"])
+        if kind == "moe":
+            E = rng.choice([1, 2, 5, 8, 16])
+            f = moe(E, rng.randint(1, min(E, 4)), rng.choice([8, 16, 40, 64]), rng.choice([0.5, 1.0, 7.0]))
+        else:
+            f = dense(rng.choice([8, 56, 128])) if kind == "dense" else None
+        layers.append((m, f))
+    return config(rng.choice([50, 131, 256]), width, layers, max_positions=rng.choice([256, 300]), eps=rng.choice([1e-5, 1e-6, 1e-3]))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(10))
+def test_drawn_configurations(seed, dtype):
+    name = f"drawn{seed}"
+    CONFIGS[name] = draw_config(seed)
+    reqs = requests(name, (1, 2, 19, 66, 150, 37), seed=seed)
+    steps, peak = mixed_steps(reqs, seed=seed, max_live=4, sizes=(1, 1, 2, 5, 16, 33, 64))
+    rows, rp = replay(name, dtype, steps, peak, page_size=(8, 16, 32)[seed % 3], max_live=4)
+    compare(name, dtype, rows, reqs)
+    assert all(g.pool.num_free == g.pool.num_pages for g in rp.runner.manager.groups), "pages were lost"
 
 
 def test_long_decoding_float32():
