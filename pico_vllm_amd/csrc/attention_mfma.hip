@@ -554,10 +554,13 @@ struct PfState {
 // rescaled only when a column of the wave outgrows that (see attend_tile).
 // krow: row 8 (col / 4) + col % 4 of the team's keys in LDS, vrow: row col of V^T at the team's keys,
 // both at this lane quarter's 16 bytes; key_pos0: position of the team's first key.
-template <int NPAIR, bool MASK, int PF_VROW, int NQB>
+// BIAS: every column has a factor of its own (c[b]: a query temperature) and a penalty on the distance to the key: the
+// exponent is s c[b] - slope log2(e) (q_pos - k_pos), which is (s + rb[b] (q_pos - k_pos)) c[b] with
+// rb = -slope log2(e) / c[b]; the penalty joins the raw score in float32 and the softmax goes on as without it.
+template <int NPAIR, bool MASK, int PF_VROW, int NQB, bool BIAS = false>
 __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow, const bf16x8 (&q)[NQB][PF_KS],
-                                          PfState (&st)[NQB], float c, int key_pos0, const int (&q_pos)[NQB],
-                                          int reach = NO_WINDOW) {
+                                          PfState (&st)[NQB], const float (&cq)[NQB], const float (&rb)[NQB], int key_pos0,
+                                          const int (&q_pos)[NQB], int reach = NO_WINDOW) {
   const int kq = (threadIdx.x & 63) >> 4;
   f32x4p s[NQB][2 * NPAIR];
   // Two query blocks a wave: the operands of a 16-key block (PF_KS reads from LDS) are requested one block ahead of
@@ -604,11 +607,14 @@ __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow
   }
 #pragma unroll
   for (int b = 0; b < NQB; b++) {
+    const float c = cq[b];
     float mx = -INFINITY;
+    const float far0 = (float)(q_pos[b] - key_pos0 - 8 * kq);   // distance to this lane's first key of the tile
 #pragma unroll
     for (int j = 0; j < 2 * NPAIR; j++)
 #pragma unroll
       for (int r = 0; r < 4; r++) {
+        if (BIAS) s[b][j][r] = fmaf(rb[b], far0 - (float)(32 * (j / 2) + 4 * (j % 2) + r), s[b][j][r]);
         if (MASK) {
           const int kpos = key_pos0 + 32 * (j / 2) + 8 * kq + 4 * (j % 2) + r;
           if (kpos > q_pos[b] || kpos <= q_pos[b] - reach) s[b][j][r] = -INFINITY;
@@ -689,12 +695,13 @@ __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow
 // NQB = 2 (one or two teams): a wave owns two blocks of 16 queries and a workgroup 128, so every K and V^T
 // operand read from LDS feeds two products; LDS traffic, which bounds the kernel when there is work for
 // every compute unit, halves per product, at the price of registers for two waves per SIMD.
-template <int KT, int NQB = 1>
+template <int KT, int NQB = 1, bool BIAS = false>
 __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefill16_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, int num_seqs, bf16_t* __restrict__ out, int nq, int nkv, int P, int num_pages,
-    float scale, int reach, int chunk_len, int max_chunks, float* __restrict__ part, const int* __restrict__ order) {
+    float scale, int reach, int chunk_len, int max_chunks, float* __restrict__ part, const int* __restrict__ order,
+    float temp_coef = 0.f, int temp_every = 0, float slope_span = 0.f) {
   static_assert(NQB == 1 || KT <= 2, "two query blocks a wave: one or two teams (three would leave a wave 170 registers)");
   constexpr int PF_TK = 64 * KT, PF_VROW = PF_TK + 8;
   constexpr int BMQ = PF_BM * NQB;            // queries per workgroup
@@ -756,6 +763,18 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   const int kv_end = chunk_len > 0 ? min(tile_kv_end, (chunk + 1) * chunk_len) : tile_kv_end;
 
   const float c = scale * 1.4426950408889634f;                 // scores go through 2^x
+  // BIAS: a column's factor grows with its position, 1 + temp_coef ln(floor((position + 1) / temp_every) + 1), and a
+  // key at distance d is penalised by slope d, slope = 2^(-slope_span (head + 1) / heads)
+  float cq[NQB], rb[NQB];
+#pragma unroll
+  for (int qb = 0; qb < NQB; qb++) {
+    cq[qb] = c;
+    rb[qb] = 0.f;
+    if (BIAS) {
+      if (temp_every > 0) cq[qb] = c * (1.0f + temp_coef * logf((float)((q_pos[qb] + 1) / temp_every + 1)));
+      if (slope_span > 0.f) rb[qb] = -exp2f(-slope_span * (float)(head + 1) / (float)nq) * 1.4426950408889634f / cq[qb];
+    }
+  }
   const int pshift = 31 - __clz(P);                            // page sizes are powers of two
   PfState st[NQB];
 #pragma unroll
@@ -791,13 +810,13 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
     if (!wave_active || key0 > wave_last_pos) return;
     if (key0 + 63 <= wave_first_pos - reach) return;            // every key lies before every query's window
     if (key0 <= wave_last_pos - reach) {                        // a window's lower edge runs through these keys
-      pf_attend<2, true, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos, reach);
+      pf_attend<2, true, PF_VROW, NQB, BIAS>(krow, vrow, qf, st, cq, rb, key0, q_pos, reach);
     } else if (key0 + 63 <= wave_first_pos) {
-      pf_attend<2, false, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos);
+      pf_attend<2, false, PF_VROW, NQB, BIAS>(krow, vrow, qf, st, cq, rb, key0, q_pos);
     } else if (key0 + 32 <= wave_last_pos) {
-      pf_attend<2, true, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos);
+      pf_attend<2, true, PF_VROW, NQB, BIAS>(krow, vrow, qf, st, cq, rb, key0, q_pos);
     } else {   // the second pair of 16-key blocks lies wholly beyond the causal frontier of this wave
-      pf_attend<1, true, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos);
+      pf_attend<1, true, PF_VROW, NQB, BIAS>(krow, vrow, qf, st, cq, rb, key0, q_pos);
     }
   };
   int ti = first_tile;
@@ -847,7 +866,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
 #pragma unroll
       for (int t = 1; t < KT; t++) M = fmaxf(M, base[(t - 1) * 4 * PER_WAVE + (PF_DT * 4) * 64]);
       const float m_use = (M == -INFINITY) ? 0.f : M;
-      const float a0 = __builtin_amdgcn_exp2f((s0.m - m_use) * c);
+      const float a0 = __builtin_amdgcn_exp2f((s0.m - m_use) * cq[qb]);
       s0.l *= a0;
       s0.m = M;                                                // what the merged sums are relative to (a chunk's part says so)
 #pragma unroll
@@ -855,7 +874,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
 #pragma unroll
       for (int t = 1; t < KT; t++) {
         const float* theirs = base + (t - 1) * 4 * PER_WAVE;
-        const float at = __builtin_amdgcn_exp2f((theirs[(PF_DT * 4) * 64] - m_use) * c);
+        const float at = __builtin_amdgcn_exp2f((theirs[(PF_DT * 4) * 64] - m_use) * cq[qb]);
         s0.l += at * theirs[(PF_DT * 4 + 1) * 64];
 #pragma unroll
         for (int tt = 0; tt < PF_DT; tt++)
@@ -1454,12 +1473,49 @@ extern "C" int pico_attn_head_dim() { return D; }
 // order (may be null): room for order_capacity >= num_tokens / 64 + num_seqs integers; with several sequences their query
 // tiles are taken longest first from the list that pf_order_kernel writes there, when order_build is set (the first
 // layer of a step) or has written there (the others: same sequences, same `teams`).
+static int attn_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                        const int* block_table, int max_pages, const int* cu_seqlens,
+                        const int* context_lens, int num_seqs, int num_tokens, void* out, int nq, int nkv,
+                        int d, int P, int num_pages, float scale, int teams, int window, int chunk_len,
+                        int max_chunks, float* part, int* order, int order_capacity, int order_build,
+                        float temp_coef, int temp_every, float slope_span, hipStream_t stream);
+
 extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int* block_table, int max_pages, const int* cu_seqlens,
                                  const int* context_lens, int num_seqs, int num_tokens, void* out, int nq, int nkv,
                                  int d, int P, int num_pages, float scale, int teams, int window, int chunk_len,
                                  int max_chunks, float* part, int* order, int order_capacity, int order_build, hipStream_t stream) {
+  return attn_prefill(q, q_stride, k_cache, v_cache, block_table, max_pages, cu_seqlens, context_lens, num_seqs, num_tokens, out,
+                      nq, nkv, d, P, num_pages, scale, teams, window, chunk_len, max_chunks, part, order, order_capacity,
+                      order_build, 0.f, 0, 0.f, stream);
+}
+
+// The same with positions in the scores: column i's scores are scaled by 1 + temp_coef ln(floor((i + 1) / temp_every) + 1)
+// (temp_every = 0: not), and a key at distance i - j costs slope_h (i - j), slope_h = 2^(-slope_span (h + 1) / nq)
+// (slope_span = 0: nothing).  Head sizes in steps of 32, whole keys (no chunks).
+extern "C" int pico_attn_prefill_scored(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                        const int* block_table, int max_pages, const int* cu_seqlens,
+                                        const int* context_lens, int num_seqs, int num_tokens, void* out, int nq, int nkv,
+                                        int d, int P, int num_pages, float scale, int teams, int window, int* order,
+                                        int order_capacity, int order_build, float temp_coef, int temp_every,
+                                        float slope_span, hipStream_t stream) {
+  PICO_REQUIRE(PICO_HEAD_DIM % 32 == 0, "pico_attn_prefill_scored: head sizes in steps of 32");
+  PICO_REQUIRE(temp_every >= 0 && slope_span >= 0.f, "pico_attn_prefill_scored: bad constants");
+  PICO_REQUIRE((uint64_t)num_pages * nkv * P * D * sizeof(bf16_t) < (1ull << 32), "pico_attn_prefill_scored: caches below 4 GiB");
+  return attn_prefill(q, q_stride, k_cache, v_cache, block_table, max_pages, cu_seqlens, context_lens, num_seqs, num_tokens, out,
+                      nq, nkv, d, P, num_pages, scale, teams, window, 0, 0, nullptr, order, order_capacity, order_build,
+                      temp_coef, temp_every, slope_span, stream);
+}
+
+static int attn_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                        const int* block_table, int max_pages, const int* cu_seqlens,
+                        const int* context_lens, int num_seqs, int num_tokens, void* out, int nq, int nkv,
+                        int d, int P, int num_pages, float scale, int teams, int window, int chunk_len,
+                        int max_chunks, float* part, int* order, int order_capacity, int order_build,
+                        float temp_coef, int temp_every, float slope_span, hipStream_t stream) {
   if (check_common("pico_attn_prefill", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
+  const bool scored = temp_every > 0 || slope_span > 0.f;
+  (void)scored;
   PICO_REQUIRE(window >= 0 && window < NO_WINDOW, "pico_attn_prefill: bad window %d", window);
   const int reach = window > 0 ? window : NO_WINDOW;
   PICO_REQUIRE(num_seqs > 0 && num_tokens >= num_seqs, "pico_attn_prefill: bad batch (%d sequences, %d tokens)", num_seqs, num_tokens);
@@ -1498,6 +1554,23 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
     }
 #define PF_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, \
                 cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach, chunk_len, max_chunks, part, ord
+    if (scored) {
+      // the same shapes of workgroup, with the columns' factors and the penalty in the scores
+#define PF_SCORED PF_ARGS, temp_coef, temp_every, slope_span
+      if (teams == 6 && PF_KT_MAX == 2)
+        prefill16_kernel<PF_KT_MAX == 2 ? 2 : 1, PF_KT_MAX == 2 ? 2 : 1, true><<<grid, 512, 0, stream>>>(PF_SCORED);
+      else if (teams == 4 && PF_KT_MAX == 2)
+        prefill16_kernel<1, PF_KT_MAX == 2 ? 2 : 1, true><<<grid, 256, 0, stream>>>(PF_SCORED);
+      else if (teams == 1 || PF_KT_MAX == 1)
+        prefill16_kernel<1, 1, true><<<grid, 256, 0, stream>>>(PF_SCORED);
+      else if (teams == 3 && PF_KT_MAX == 2)
+        prefill16_kernel<PF_KT_MAX == 2 ? 3 : 1, 1, true><<<grid, 768, 0, stream>>>(PF_SCORED);
+      else
+        prefill16_kernel<PF_KT_MAX, 1, true><<<grid, 256 * PF_KT_MAX, 0, stream>>>(PF_SCORED);
+#undef PF_SCORED
+      PICO_LAUNCH_CHECK();
+      return 0;
+    }
     if (teams == 6 && PF_KT_MAX == 2)             // 128 queries a workgroup and two key teams
       prefill16_kernel<PF_KT_MAX == 2 ? 2 : 1, PF_KT_MAX == 2 ? 2 : 1><<<grid, 512, 0, stream>>>(PF_ARGS);
     else if (teams == 4 && PF_KT_MAX == 2)        // 128 queries a workgroup, two blocks of 16 a wave

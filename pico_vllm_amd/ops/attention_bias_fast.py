@@ -7,11 +7,13 @@ from typing import Optional
 import torch
 
 from . import library
+from . import attention_fast
 from .attention_fast import compute_units
 from .kernels import KernelError, _check, _check_cache2, _ptr, _stream
 
 c_float = ctypes.c_float
 MAX_CHUNKS = 32
+PROMPT_KERNEL_FROM = 64      # tokens of a step from which the prompt kernel serves it (a tile of its workgroups)
 
 
 def supported(key_dim: int, value_dim: int) -> bool:
@@ -28,6 +30,11 @@ class FastBiasAttention:
         if self.lib.pico_attnb_key_dim() != key_dim or self.lib.pico_attnb_value_dim() != value_dim:
             raise KernelError("attention library was built for other sizes")
         self.cus = compute_units()
+        # keys and values of one size in steps of 32: prompt steps go through the rotary attention's prompt kernel (keys
+        # staged in LDS for 64 or 128 queries), which takes the columns' factors and the penalty into its scores
+        self.tuned = None
+        if key_dim == value_dim and key_dim % 32 == 0 and attention_fast.supported(nq, nkv, key_dim, window):
+            self.tuned = attention_fast.FastAttention(nq, nkv, key_dim, window)
 
     def split(self, num_tokens: int) -> bool:
         """Whether the four waves of a workgroup share ONE block of 16 query columns (few blocks: the chip is filled
@@ -47,8 +54,23 @@ class FastBiasAttention:
         blocks = (-(-num_tokens // max(1, 16 // R)) + num_seqs) * -(-R // 16) * self.nkv
         return max(1, min(MAX_CHUNKS, -(-2 * self.cus // blocks)))
 
+    def prompt_shape(self, ctx) -> int:
+        """The shape of the prompt kernel's workgroups for this step (0: that kernel does not serve it)."""
+        if self.tuned is None or ctx.num_tokens < PROMPT_KERNEL_FROM:
+            return 0
+        key = ("bias_attention_shape", self.nq, self.nkv, self.dk, self.window)
+        if key not in ctx.shared:
+            shape = 1
+            if "cu_seqlens" in ctx.host and "context_lens" in ctx.host:
+                B = ctx.num_seqs
+                cu = ctx.host["cu_seqlens"]
+                real = B - int(ctx.host.get("filler", 0))         # the filler behind a recorded portion does not count
+                shape = int(self.tuned.prefill_teams((cu[1:B + 1] - cu[:B])[:real], ctx.host["context_lens"][:real]))
+            ctx.shared[key] = shape
+        return ctx.shared[key]
+
     def plan(self, ctx) -> tuple:
-        return (bool(self.split(ctx.num_tokens)), self.chunks(ctx.num_tokens, ctx.num_seqs))
+        return (bool(self.split(ctx.num_tokens)), self.chunks(ctx.num_tokens, ctx.num_seqs), self.prompt_shape(ctx))
 
     def run(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, positions, num_seqs: int,
             split: Optional[bool] = None, out: Optional[torch.Tensor] = None, chunks: Optional[int] = None) -> torch.Tensor:
@@ -87,8 +109,20 @@ class FastBiasAttention:
         return out
 
     def __call__(self, qkv, cache, block_table, ctx):
+        split, chunks, shape = self.plan(ctx)
+        if shape and cache.k.numel() * cache.k.element_size() < (1 << 32):
+            B = ctx.num_seqs
+            order, build = None, False
+            if B >= 2:      # several sequences: the list of their query tiles, longest first, written by the first layer
+                key = ("bias_attention_order", self.dk, shape)
+                order, build = ctx.shared.get(key), key not in ctx.shared
+                if build:
+                    order = ctx.shared[key] = self.tuned.order_list(qkv.shape[0], B, qkv.device)
+            return self.tuned.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, B, self.scale,
+                                      teams=shape, order=order, order_build=build,
+                                      scored=(self.temp_coef, self.temp_every, self.slope_span))
         return self.run(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.positions, ctx.num_seqs,
-                        split=self.plan(ctx)[0], chunks=self.plan(ctx)[1])
+                        split=split, chunks=chunks)
 
 
 def choose(mixer) -> Optional[FastBiasAttention]:

@@ -144,7 +144,8 @@ class FastAttention:
 
     def prefill(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, context_lens, num_seqs: int,
                 scale: float, out: Optional[torch.Tensor] = None, teams: int = 0, chunk_len: int = 0,
-                max_chunks: int = 0, order: Optional[torch.Tensor] = None, order_build: bool = True) -> torch.Tensor:
+                max_chunks: int = 0, order: Optional[torch.Tensor] = None, order_build: bool = True,
+                scored: Optional[tuple] = None) -> torch.Tensor:
         """q [T, >= nq*d] bfloat16 (row stride free); any mixture of portions; returns [T, nq*d].
         teams: 0 lets the kernel choose, else the result of ``prefill_teams``.  chunk_len > 0: the keys of every
         query tile are cut into chunks of that many, each a workgroup of its own (``max_chunks`` of them cover the
@@ -158,6 +159,18 @@ class FastAttention:
         self._check_meta(block_table, cu_seqlens, num_seqs + 1, context_lens, num_seqs)
         if out is None:
             out = torch.empty(T, nq * d, dtype=torch.bfloat16, device=q.device)
+        if scored is not None:
+            # positions in the scores: (temp_coef, temp_every, slope_span), a factor that grows with the query's position
+            # and a penalty on the distance to the key; whole keys only
+            temp_coef, temp_every, slope_span = scored
+            if d % 32 or chunk_len or k_cache.numel() * k_cache.element_size() >= (1 << 32):
+                raise KernelError("scored prefill: head sizes in steps of 32, whole keys, caches below 4 GiB")
+            _check(self.lib, self.lib.pico_attn_prefill_scored(
+                _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+                _ptr(cu_seqlens), _ptr(context_lens), num_seqs, T, _ptr(out), nq, nkv, d, P, pages, c_float(scale),
+                teams, self.window, _ptr(order), 0 if order is None else order.numel(), 1 if order_build else 0,
+                c_float(temp_coef), int(temp_every), c_float(slope_span), _stream()))
+            return out
         part = None
         if chunk_len and k_cache.numel() * k_cache.element_size() >= (1 << 32):
             chunk_len = max_chunks = 0          # the kernel that cuts keys into chunks addresses the cache with 32 bits

@@ -48,9 +48,14 @@ CONFIGS = {
     "c": config(61, 72, [(attention(3, 1, 24, 40, 5, (0.5, 3), True), dense(100)),
                          (attention(3, 1, 24, 40, 64, (0.5, 3), True), moe(3, 2, 24, 1.0))]),
     # sizes the matrix-core kernels take (multiples of 32), a window that spans pages, many heads a group
-    "d": config(256, 128, [(attention(8, 1, 64, 32, 40, (0.5, 16), True), dense(256)),
-                           (attention(8, 1, 64, 32, 40, (0.5, 16), True), moe(16, 2, 64, 1.0)),
+    "d": config(256, 128, [(attention(8, 1, 64, 32, 44, (0.6, 16), True), dense(256)),
+                           (attention(8, 1, 64, 32, 44, (0.6, 16), True), moe(12, 2, 64, 1.0)),
                            (attention(8, 2, 32, 64, 100, None, False), moe(4, 4, 32, 3.0))], max_positions=1024),
+    # keys and values of one size in steps of 32 (prompt steps take another kernel), windowed and not, with and without
+    # a temperature
+    "e": config(200, 96, [(attention(6, 2, 32, 32, 24, (0.8, 10), True), dense(96)),
+                          (attention(6, 2, 32, 32, None, None, True), moe(6, 2, 32, 1.5)),
+                          (attention(4, 4, 64, 64, 70, (0.5, 64), False), None)], max_positions=600),
 }
 
 

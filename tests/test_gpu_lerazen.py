@@ -168,6 +168,9 @@ ATTN_CASES = [
     (5, 1, 64, 64, 33, None, 16, 31, 34),           # heads a group that do not divide 16
     (4, 2, 64, 32, None, (0.3, 100), 16, 1500, 2),  # many keys: pieces of several turns of the waves
     (4, 2, 64, 32, 700, None, 16, 1203, 1),
+    (4, 2, 32, 32, 50, (0.6, 9), 16, 200, 150),     # keys and values of one size: the prompt kernel too
+    (6, 2, 128, 128, None, (0.4, 32), 16, 70, 300),
+    (2, 1, 64, 64, 130, None, 8, 0, 260),
 ]
 
 
@@ -198,6 +201,12 @@ def test_attention_kernels(case, dtype):
         for split, chunks in ((False, 1), (True, 1), (True, 2), (True, 3), (True, 32)):
             got = fast.run(qd, K, V, bt, cu, pos, 1, split=split, chunks=chunks)
             assert torch.allclose(got.cpu().double().view(new, H, dv), want, atol=tol, rtol=tol), f"split={split} chunks={chunks}"
+        if fast.tuned is not None:
+            # the prompt kernel with the positions in its scores, in every shape of workgroup
+            cl = torch.tensor([N], dtype=torch.int32, device=DEV)
+            for shape in (1, 2, 3, 4, 6):
+                got = fast.tuned.prefill(qd, K, V, bt, cu, cl, 1, scale, teams=shape, scored=(tc, te, 8.0))
+                assert torch.allclose(got.cpu().double().view(new, H, dv), want, atol=tol, rtol=tol), f"prompt kernel, shape {shape}"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -396,7 +405,7 @@ def test_learned_positions_are_added_in_float32():
 # ---------------------------------------------------------------------------------------------------------------
 # the model in the engine
 # ---------------------------------------------------------------------------------------------------------------
-LENGTHS = {"a": (1, 2, 45, 130), "b": (3, 77, 150), "c": (1, 29, 90), "d": (5, 64, 233)}
+LENGTHS = {"a": (1, 2, 45, 130), "b": (3, 77, 150), "c": (1, 29, 90), "d": (5, 64, 233), "e": (2, 64, 65, 310)}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
