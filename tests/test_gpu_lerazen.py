@@ -569,3 +569,56 @@ def test_greedy_generation_through_the_entry_point(dtype, graphs):
                 assert gap < (1e-4 if dtype == "float32" else 0.1), f"token {tok} instead of {best}, gap {gap}"
             seq.append(tok)
     llm.engine.runner.manager.check()
+
+
+def test_command_line_generates_from_a_model_folder(capsys):
+    """python -m pico_vllm_amd.run on a Lerazen folder: the architecture is found from config.json, sampling with a
+    temperature and a seed gives the same tokens twice."""
+    from pico_vllm_amd import run
+    common = ["--model", model_dir("e"), "--prompt-ids", "5,17,3", "--prompt-ids", "9", "--max-new-tokens", "6", "--ignore-eos",
+              "--num-gpu-blocks", "16", "--max-seq-len", "64"]
+    assert run.main(common + ["--dtype", "float32"]) == 0
+    lines = [l for l in capsys.readouterr().out.splitlines() if l.startswith("[")]
+    assert len(lines) == 2 and all(len(l.split(")")[1].split()) == 6 for l in lines)
+    seq = [5, 17, 3]
+    for tok in map(int, lines[0].split(")")[1].split()):
+        lg = plain_logits("e", seq)[-1]
+        assert lg[tok] >= lg.max() - 1e-4 * lg.std()          # the plain argmax (or its equal within rounding)
+        seq.append(tok)
+    runs = []
+    for _ in range(2):
+        assert run.main(common + ["--dtype", "bfloat16", "--temperature", "0.9", "--top-p", "0.8", "--seed", "7"]) == 0
+        runs.append([l for l in capsys.readouterr().out.splitlines() if l.startswith("[")])
+    assert runs[0] == runs[1]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_replay_program_in_a_subprocess(dtype):
+    import json
+    import os
+    import subprocess
+    import tempfile
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    name = "c"
+    reqs = requests(name, (30, 9, 75), seed=8)
+    steps, peak = mixed_steps(reqs, seed=5, max_live=2)
+    lines = [json.dumps({"step": k, "entries": [{"id": r, "tokens": t, "want": list(w)} for r, t, w in entries], "end": list(end)})
+             for k, (entries, end) in enumerate(steps)]
+    with tempfile.TemporaryDirectory() as out:
+        r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", model_dir(name), "--dtype", dtype, "--out", out,
+                            "--max-tokens", str(peak)], input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
+        assert r.returncode == 0, r.stderr[-2000:]
+        assert [l for l in r.stdout.split("\n") if l.startswith("done")] == [f"done {k}" for k in range(len(steps))]
+        rows, fed = {}, {}
+        for k, (entries, end) in enumerate(steps):
+            wanted = sum(len(w) for _, _, w in entries)
+            a = np.fromfile(os.path.join(out, f"{k}.f32"), dtype="<f4").reshape(wanted, -1)
+            at = 0
+            for rid, t, w in entries:
+                for x in w:
+                    rows[(rid, fed.get(rid, 0) + x)] = a[at]
+                    at += 1
+                fed[rid] = fed.get(rid, 0) + len(t)
+            for rid in end:
+                fed.pop(rid, None)
+    compare(name, dtype, rows, reqs)
