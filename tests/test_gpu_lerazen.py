@@ -159,8 +159,8 @@ ATTN_CASES = [
     # H, G, dk, dv, window, temp, page, prefix, new
     (4, 2, 32, 16, 12, (0.7, 8), 16, 0, 37),
     (4, 2, 32, 16, 12, (0.7, 8), 16, 30, 1),
-    (8, 1, 64, 32, 40, (0.5, 16), 16, 100, 23),
-    (8, 1, 64, 32, 40, None, 8, 131, 1),
+    (8, 1, 64, 32, 44, (0.6, 16), 16, 100, 23),
+    (8, 1, 64, 32, 44, None, 8, 131, 1),
     (6, 6, 32, 48, None, (1.1, 16), 16, 300, 5),
     (6, 6, 32, 48, None, None, 32, 517, 1),
     (3, 1, 24, 40, 5, (0.5, 3), 8, 9, 11),
@@ -319,7 +319,7 @@ def test_routed_experts(sizes, dtype):
 
 @pytest.mark.parametrize("grouped", [False, True])
 @pytest.mark.parametrize("sizes", [(1, 6, 1, 8, 8), (3, 4, 2, 72, 40), (20, 3, 3, 104, 136), (500, 8, 2, 192, 256),
-                                   (130, 40, 1, 64, 64)])
+                                   (130, 40, 1, 64, 64), (1500, 64, 4, 96, 256), (2000, 3, 1, 64, 136)])
 def test_expert_kernels_agree(sizes, grouped):
     """Both bfloat16 paths (rows that stream their expert's matrices; rows sorted by expert for the matrix cores) against
     the plain kernel, with experts that get no row, one row, and more rows than a tile holds."""
