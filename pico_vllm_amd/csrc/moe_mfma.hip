@@ -45,6 +45,12 @@ __device__ __forceinline__ uint4 scale8(const uint4& v, float w) {
   return o;
 }
 
+// v where keep, else zeros (component by component: the values stay in registers)
+__device__ __forceinline__ uint4 keep8(const uint4& v, bool keep) {
+  const uint32_t m = keep ? 0xffffffffu : 0u;
+  return make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+}
+
 __device__ __forceinline__ float dot8(const uint4& a, const float* x, float acc) {
   float f[8];
   unpack8(a, f);
@@ -261,9 +267,10 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
 #pragma unroll
   for (int r = 0; r < 16; r++) { acc00[r] = 0.f; acc01[r] = 0.f; acc10[r] = 0.f; acc11[r] = 0.f; }
 
-  const uint4 zero = make_uint4(0, 0, 0, 0);
   uint4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
-  // K is a multiple of 8: the 8 k of a load are in or out together; a load beyond K reads k = 0 .. and is cleared
+  // K is a multiple of 8: the 8 k of a load are in or out together; a load beyond K reads k = 0 .. instead.  What must
+  // read as zero (rows that do not exist, k beyond K) is cleared where the stage is written to LDS, not here: a select
+  // on a register that a load has just been asked for would wait for that load in front of the products
 #define MOE_FETCH(k0)                                                      \
   {                                                                        \
     const bool k_ok = (k0) + sk < K;                                       \
@@ -276,14 +283,6 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
     rb1 = *reinterpret_cast<const uint4*>(b_src1 + ko);                    \
     rb2 = *reinterpret_cast<const uint4*>(b_src2 + ko);                    \
     rb3 = *reinterpret_cast<const uint4*>(b_src3 + ko);                    \
-    if (!(a_ok0 && k_ok)) ra0 = zero;                                      \
-    if (!(a_ok1 && k_ok)) ra1 = zero;                                      \
-    if (!(a_ok2 && k_ok)) ra2 = zero;                                      \
-    if (!(a_ok3 && k_ok)) ra3 = zero;                                      \
-    if (!(b_ok0 && k_ok)) rb0 = zero;                                      \
-    if (!(b_ok1 && k_ok)) rb1 = zero;                                      \
-    if (!(b_ok2 && k_ok)) rb2 = zero;                                      \
-    if (!(b_ok3 && k_ok)) rb3 = zero;                                      \
   }
   MOE_FETCH(0)
   const int frag = (lane & 31) * MOE_LD + (lane >> 5) * 8;    // a lane's place in a block of 32 rows
@@ -295,14 +294,15 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
     {
       bf16_t* as = As + srow * MOE_LD + sk;
       bf16_t* bs = Bs + srow * MOE_LD + sk;
-      *reinterpret_cast<uint4*>(as) = UP ? scale8(ra0, a_w0) : ra0;
-      *reinterpret_cast<uint4*>(as + 32 * MOE_LD) = UP ? scale8(ra1, a_w1) : ra1;
-      *reinterpret_cast<uint4*>(as + 64 * MOE_LD) = UP ? scale8(ra2, a_w2) : ra2;
-      *reinterpret_cast<uint4*>(as + 96 * MOE_LD) = UP ? scale8(ra3, a_w3) : ra3;
-      *reinterpret_cast<uint4*>(bs) = rb0;
-      *reinterpret_cast<uint4*>(bs + 32 * MOE_LD) = rb1;
-      *reinterpret_cast<uint4*>(bs + 64 * MOE_LD) = rb2;
-      *reinterpret_cast<uint4*>(bs + 96 * MOE_LD) = rb3;
+      const bool k_in = k0 + sk < K;
+      *reinterpret_cast<uint4*>(as) = keep8(UP ? scale8(ra0, a_w0) : ra0, a_ok0 && k_in);
+      *reinterpret_cast<uint4*>(as + 32 * MOE_LD) = keep8(UP ? scale8(ra1, a_w1) : ra1, a_ok1 && k_in);
+      *reinterpret_cast<uint4*>(as + 64 * MOE_LD) = keep8(UP ? scale8(ra2, a_w2) : ra2, a_ok2 && k_in);
+      *reinterpret_cast<uint4*>(as + 96 * MOE_LD) = keep8(UP ? scale8(ra3, a_w3) : ra3, a_ok3 && k_in);
+      *reinterpret_cast<uint4*>(bs) = keep8(rb0, b_ok0 && k_in);
+      *reinterpret_cast<uint4*>(bs + 32 * MOE_LD) = keep8(rb1, b_ok1 && k_in);
+      *reinterpret_cast<uint4*>(bs + 64 * MOE_LD) = keep8(rb2, b_ok2 && k_in);
+      *reinterpret_cast<uint4*>(bs + 96 * MOE_LD) = keep8(rb3, b_ok3 && k_in);
     }
     __syncthreads();
     if (k0 + MOE_BK < K) MOE_FETCH(k0 + MOE_BK)               // the next stage travels while this one is multiplied
