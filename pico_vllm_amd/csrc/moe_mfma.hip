@@ -304,8 +304,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
       *reinterpret_cast<uint4*>(bs + 64 * MOE_LD) = keep8(rb2, b_ok2 && k_in);
       *reinterpret_cast<uint4*>(bs + 96 * MOE_LD) = keep8(rb3, b_ok3 && k_in);
     }
-    __syncthreads();
     if (k0 + MOE_BK < K) MOE_FETCH(k0 + MOE_BK)               // the next stage travels while this one is multiplied
+    __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < MOE_BK; ks += 16) {
       const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(As + a_off + ks);
