@@ -51,6 +51,8 @@ struct TileRows {
 #define EPI_F32 1      // out float32 [M, N] (slab `blockIdx.y` when the k range is split over the grid)
 #define EPI_SWIGLU 2   // W = [gate rows; up rows], out bf16 [M, N / 2]
 #define EPI_RELU2 3    // out bf16 [M, N] = max(x W^T + bias, 0)^2
+#define EPI_F32_ADD 4  // out float32 [M, N] += x W^T + bias (a residual stream; the k range is not split over the grid, so
+                       // every element has one writer)
 #define MAX_SK_SLABS 8 // partial sums that a norm in front of a projection adds up
 
 // The sums of one output tile when K is no multiple of 64 (any multiple of 8): operands go through
@@ -347,6 +349,11 @@ __device__ __forceinline__ void skinny_finish(float (*red)[MT][16][64], int tile
 #pragma unroll
         for (int b = 0; b < 4; b++)
           if (t0 + b < rows && n + b < N) o[b] = v[b];
+      } else if (EPI == EPI_F32_ADD) {
+        float* o = (float*)out + (size_t)m * ldo + n;
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+          if (t0 + b < rows && n + b < N) o[b] += v[b];
       } else {
         bf16_t* o = (bf16_t*)out + (size_t)m * ldo + n;
 #pragma unroll
@@ -655,7 +662,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   PICO_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K,
                "pico_gemm_skinny: K and the row strides must be multiples of 8 (K=%d ldx=%d ldw=%d)", K, ldx, ldw);
   PICO_REQUIRE((uintptr_t)X % 16 == 0 && (uintptr_t)W % 16 == 0, "pico_gemm_skinny: operands must be 16-byte aligned");
-  PICO_REQUIRE(epilogue >= 0 && epilogue <= 3, "pico_gemm_skinny: unknown epilogue %d", epilogue);
+  PICO_REQUIRE(epilogue >= 0 && epilogue <= 4, "pico_gemm_skinny: unknown epilogue %d", epilogue);
   PICO_REQUIRE(k_splits >= 1 && (k_splits == 1 || epilogue == EPI_F32), "pico_gemm_skinny: only the float32 epilogue can split k over the grid");
   PICO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && bias == nullptr), "pico_gemm_skinny: SwiGLU needs an even N and no bias");
   const int n_out = epilogue == EPI_SWIGLU ? N / 2 : N;
@@ -687,6 +694,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
     if (epilogue == EPI_BF16) LAUNCHP(EPI_BF16);
     else if (epilogue == EPI_F32) LAUNCHP(EPI_F32);
     else if (epilogue == EPI_RELU2) LAUNCHP(EPI_RELU2);
+    else if (epilogue == EPI_F32_ADD) LAUNCHP(EPI_F32_ADD);
     else LAUNCHP(EPI_SWIGLU);
 #undef LAUNCHP
     PICO_LAUNCH_CHECK();
@@ -718,6 +726,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   if (epilogue == EPI_BF16) LAUNCH(EPI_BF16);
   else if (epilogue == EPI_F32) LAUNCH(EPI_F32);
   else if (epilogue == EPI_RELU2) LAUNCH(EPI_RELU2);
+  else if (epilogue == EPI_F32_ADD) LAUNCH(EPI_F32_ADD);
   else LAUNCH(EPI_SWIGLU);
 #undef LAUNCH4
 #undef LAUNCH

@@ -212,7 +212,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
     return out
 
 
-EPI_BF16, EPI_F32, EPI_SWIGLU, EPI_RELU2 = 0, 1, 2, 3
+EPI_BF16, EPI_F32, EPI_SWIGLU, EPI_RELU2, EPI_F32_ADD = 0, 1, 2, 3, 4
 MAX_HEAD_DIM = 256          # the largest head size any attention kernel takes
 
 
@@ -240,10 +240,11 @@ def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_BF16,
-                k_splits: int = 1) -> torch.Tensor:
+                k_splits: int = 1, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [M <= 64, K] x w [N, K]^T, both bfloat16.  EPI_BF16 -> bf16 [M, N]; EPI_F32 -> float32 [M, N], or with
     k_splits > 1 a stack [k_splits, M, N] of partial sums (bias in the first); EPI_SWIGLU (w = [gate; up])
-    -> bf16 [M, N / 2] = silu(gate) * up; EPI_RELU2 -> bf16 [M, N] = max(x w^T + bias, 0)^2."""
+    -> bf16 [M, N / 2] = silu(gate) * up; EPI_RELU2 -> bf16 [M, N] = max(x w^T + bias, 0)^2; EPI_F32_ADD: ``out``
+    (contiguous float32 [M, N], a residual stream) += x w^T + bias, every element by one writer."""
     _gpu(a, w, bias)
     M, K = a.shape
     N, K2 = w.shape
@@ -255,7 +256,13 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
         raise KernelError("gemm_skinny: bias must be contiguous float32 [N]")
     if k_splits > 1 and epilogue != EPI_F32:
         raise KernelError("gemm_skinny: only the float32 epilogue can leave partial sums")
-    if epilogue == EPI_F32:
+    if epilogue == EPI_F32_ADD:
+        if out is None or out.dtype != torch.float32 or tuple(out.shape) != (M, N) or not out.is_contiguous() or not out.is_cuda:
+            raise KernelError(f"gemm_skinny: adding needs a contiguous float32 [{M}, {N}] to add into")
+        ldo = N
+    elif out is not None:
+        raise KernelError("gemm_skinny: only the adding epilogue takes an output")
+    elif epilogue == EPI_F32:
         shape = (M, N) if k_splits == 1 else (k_splits, M, N)
         out = torch.empty(shape, dtype=torch.float32, device=a.device)
         ldo = N

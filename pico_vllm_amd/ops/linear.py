@@ -124,6 +124,13 @@ class Linear:
         y = self(x)
         return kernels.relu2(y, out=y)
 
+    def add_into(self, x: torch.Tensor, resid: torch.Tensor) -> torch.Tensor:
+        """resid (float32 [T, N], in place) += x W^T + b.  With few rows the sum is the epilogue of the weight-streaming
+        kernel; otherwise the product and then the sum."""
+        if self.weight.dtype == torch.bfloat16 and kernels.skinny_ok(x, self.weight):
+            return kernels.gemm_skinny(x, self.weight, self.bias_f32, kernels.EPI_F32_ADD, out=resid)
+        return kernels.residual_add(resid, self(x))
+
     def partial(self, x: torch.Tensor) -> torch.Tensor:
         """x W^T as something a norm's ``add_norm`` takes as delta: [T, N], or, when the matrix is
         too small to fill the chip with one workgroup per output tile, a float32 stack [S, T, N] of

@@ -113,6 +113,14 @@ class DistanceBiasAttention(Mixer):
         return own + super().graph_variant(ctx)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
+        return self.o(self.attend(x, ctx, cache))
+
+    def forward_into(self, x: torch.Tensor, ctx: StepContext, cache, resid: torch.Tensor) -> None:
+        """resid += the mixer's output: with few rows the sum is the epilogue of the output projection."""
+        self.o.add_into(self.attend(x, ctx, cache), resid)
+
+    def attend(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
+        """The heads' outputs [T, H dv] in front of the output projection."""
         bt = ctx.block_tables[cache.group]
         if getattr(cache, "read_only", False):
             # another run's keys and values: nothing is stored, every token's slot reads as "none"
@@ -136,4 +144,4 @@ class DistanceBiasAttention(Mixer):
             a = kernels.attn_bias_plain(qkv, cache.k, cache.v, bt, ctx.positions, ctx.token_seq, self.nq, self.nkv,
                                         self.dk, self.dv, self.scale, self.window, self.temp_coef, self.temp_every,
                                         self.slope_span)
-        return self.o(a)
+        return a

@@ -47,13 +47,18 @@ class PreNormBlock(Block):
 class ParallelBlock(Block):
     """h = norm1(x); x += mixer(h) + ff(h): one norm, and both sublayers read its output.  A layer without a
     feed-forward names the part "none" in that slot.  The sums are float32: the mixer's output joins the residual stream
-    at once, the feed-forward's is handed on as ``pending`` and the next norm adds it."""
+    at once (a mixer with ``forward_into(h, ctx, cache, resid)`` adds it itself, as the last step of its output
+    projection), the feed-forward's is handed on as ``pending`` and the next norm adds it."""
     slot_categories = {"norm1": "norm", "mixer": "mixer", "ff": "feed_forward"}
     graph_safe_prompts = True
 
     def forward(self, resid, pending, ctx, cache):
         p = self.parts
         h = p["norm1"].add_norm(resid, pending)
+        into = getattr(p["mixer"], "forward_into", None)
+        if into is not None:
+            into(h, ctx, cache, resid)                         # the mixer adds its output to the stream itself
+            return resid, p["ff"].forward(h, ctx)
         a = p["mixer"].forward(h, ctx, cache)
         f = p["ff"].forward(h, ctx)
         if f is None:

@@ -622,3 +622,24 @@ def test_the_replay_program_in_a_subprocess(dtype):
             for rid in end:
                 fed.pop(rid, None)
     compare(name, dtype, rows, reqs)
+
+
+@pytest.mark.parametrize("rows", [1, 5, 33, 64, 300])
+@pytest.mark.parametrize("sizes", [(96, 64), (1536, 1536), (200, 72)])
+def test_projection_adds_into_the_stream(rows, sizes):
+    """resid += x W^T + b: as the epilogue of the weight-streaming kernel for few rows, product and sum otherwise."""
+    from pico_vllm_amd.ops.linear import Linear
+    N, K = sizes
+    g = torch.Generator().manual_seed(rows + N)
+    w = (torch.randn(N, K, generator=g) * K ** -0.5).bfloat16()
+    b = torch.randn(N, generator=g) * 0.1
+    x = torch.randn(rows, K, generator=g).bfloat16()
+    resid = torch.randn(rows, N, generator=g) * 3
+    lin = Linear(w.to(DEV), b.to(DEV))
+    got = resid.clone().to(DEV)
+    assert lin.add_into(x.to(DEV), got) is got
+    want = resid.double() + x.double() @ w.double().t() + b.double()
+    assert torch.allclose(got.cpu().double(), want, atol=2e-2, rtol=2e-2)
+    # few rows: only the product's own float32 rounding stands between the two
+    if rows <= 64:
+        assert float((got.cpu().double() - want).abs().max()) < 1e-4 * max(1.0, float(want.abs().max()))
