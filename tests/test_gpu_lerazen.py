@@ -171,6 +171,9 @@ ATTN_CASES = [
     (4, 2, 32, 32, 50, (0.6, 9), 16, 200, 150),     # keys and values of one size: the prompt kernel too
     (6, 2, 128, 128, None, (0.4, 32), 16, 70, 300),
     (2, 1, 64, 64, 130, None, 8, 0, 260),
+    (3, 1, 96, 96, 60, (0.9, 20), 16, 50, 140),
+    (2, 2, 160, 160, None, (0.2, 50), 16, 33, 100),
+    (2, 1, 256, 256, 90, None, 16, 120, 70),
 ]
 
 
