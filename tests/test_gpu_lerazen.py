@@ -510,7 +510,7 @@ def draw_config(seed):
     """A configuration drawn at random: sizes, head counts, windows, constants and the order of layers all differ from
     the hand-picked ones, and include the values that make mechanisms vanish (a window of 1, one expert, one head)."""
     rng = random.Random(1000 + seed)
-    width = rng.choice([24, 40, 64, 72, 96, 128])
+    width = rng.choice([24, 40, 64, 72, 90, 96, 100, 128])           # also widths that are no multiple of 8, or of 4
     kv_heads, vdim = rng.choice([1, 2, 3]), rng.choice([8, 16, 24, 32, 48, 64])      # the same in all layers that mix values
     layers = []
     for _ in range(rng.randint(1, 5)):
@@ -522,7 +522,7 @@ def draw_config(seed):
         kind = rng.choice(["none", "dense", "moe", "moe"])
         if kind == "moe":
             E = rng.choice([1, 2, 5, 8, 16])
-            f = moe(E, rng.randint(1, min(E, 4)), rng.choice([8, 16, 40, 64]), rng.choice([0.5, 1.0, 7.0]))
+            f = moe(E, rng.randint(1, min(E, 4)), rng.choice([8, 12, 16, 40, 64]), rng.choice([0.5, 1.0, 7.0]))
         else:
             f = dense(rng.choice([8, 56, 128])) if kind == "dense" else None
         layers.append((m, f))
