@@ -33,6 +33,10 @@ class CacheGroup:
     def window(self) -> int:
         return self.spec.window
 
+    @property
+    def keep_first(self) -> int:
+        return self.spec.keep_first
+
 
 @dataclass
 class RequestCache:
@@ -132,7 +136,8 @@ class CacheManager:
     def advance(self, req: Hashable, num_computed: int) -> None:
         """Record that positions [0, num_computed) are cached, and give back
         the pages that every window has passed: the next query sits at
-        position num_computed or later and reads keys > position - window."""
+        position num_computed or later and reads keys > position - window.  Pages that
+        hold any of a group's first ``keep_first`` positions are never given back early."""
         rc = self.requests[req]
         rc.num_computed = num_computed
         for gi, g in enumerate(self.groups):
@@ -142,6 +147,8 @@ class CacheManager:
             if first_needed <= 0:
                 continue
             dead_upto = min(first_needed // self.page_size, len(rc.tables[gi]))
+            if rc.first_live[gi] == 0:
+                rc.first_live[gi] = min(_cdiv(g.keep_first, self.page_size), len(rc.tables[gi]))   # these pages stay
             gone = [rc.tables[gi][j] for j in range(rc.first_live[gi], dead_upto)]
             for j in range(rc.first_live[gi], dead_upto):
                 rc.tables[gi][j] = -1

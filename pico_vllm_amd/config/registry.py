@@ -20,13 +20,17 @@ class Architecture:
     # for reports and measurements, so that the programs that make them read no architecture's keys:
     sizes: Optional[Callable[[Any], Dict[str, Any]]] = None          # typed config -> flat {name: number} of its sizes
     with_layers: Optional[Callable[[Dict[str, Any], int], Dict[str, Any]]] = None   # raw config, n -> the same layer sizes, n layers
+    # True: config_from_dict takes a second argument, {tensor name: shape} of the checkpoint (or None where there is
+    # none yet), for sizes that config.json leaves to the tensors
+    reads_shapes: bool = False
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, config_from_dict, build_spec, sizes=None, with_layers=None) -> Architecture:
-    arch = Architecture(name, config_from_dict, build_spec, sizes, with_layers)
+def register_architecture(name: str, config_from_dict, build_spec, sizes=None, with_layers=None,
+                          reads_shapes: bool = False) -> Architecture:
+    arch = Architecture(name, config_from_dict, build_spec, sizes, with_layers, reads_shapes)
     _ARCHITECTURES[name] = arch
     return arch
 
@@ -53,5 +57,19 @@ def load_model_description(model_dir: str):
     """(architecture, typed config, ModelSpec) of a model folder."""
     raw = read_config_json(model_dir)
     arch = resolve_architecture(raw)
-    cfg = arch.config_from_dict(raw)
+    if arch.reads_shapes:
+        cfg = arch.config_from_dict(raw, checkpoint_shapes(model_dir))
+    else:
+        cfg = arch.config_from_dict(raw)
     return arch, cfg, arch.build_spec(cfg)
+
+
+def checkpoint_shapes(model_dir: str) -> Dict[str, tuple]:
+    """{tensor name: shape} from the headers of the folder's safetensors files (no tensor is read)."""
+    from ..weights.safetensors_io import SafetensorsFile, list_safetensors
+    out: Dict[str, tuple] = {}
+    for path in list_safetensors(model_dir):
+        with SafetensorsFile(path) as sf:
+            for name, (_, shape) in sf.entries.items():
+                out[name] = tuple(shape)
+    return out

@@ -5,6 +5,9 @@
 //   s_ij = (q_i . k_j) * scale * temp(i) - slope_h * (i - j),   keys j <= i, with a window only i - j < window
 //   temp(i) = 1 + coef * ln(floor((i + 1) / every) + 1)         (every == 0: 1)
 //   slope_h = 2^(-span * (h + 1) / nq)                          (span == 0: no penalty)
+//   optionally s_ij <- cap * tanh(s_ij / cap); with a window, the first `keep_first` positions of a sequence stay
+//   visible to every later query (at their true distance); optionally o_i is multiplied element by element with
+//   sigmoid(gate_i) before it is written
 //   softmax over the visible keys, o_i = sum_j p_ij v_j
 //
 // A page holds k as [kv heads, page, dk] and v as [kv heads, dv, page].  Scores, softmax and the sums over keys are
@@ -15,6 +18,8 @@
 struct BiasParams {
   float scale, temp_coef, slope_span;
   int temp_every, window;
+  float softcap;      // 0: none
+  int keep_first;     // with a window: keys below this position are seen whatever their distance
 };
 
 __device__ __forceinline__ float query_scale(const BiasParams& p, int pos) {
@@ -91,7 +96,7 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ positions,
     const int* __restrict__ token_seq, T* __restrict__ out, int nq, int nkv, int dk, int dv, int P, BiasParams bp,
-    int num_pages) {
+    int num_pages, const T* __restrict__ gate, int gate_stride) {
   extern __shared__ float lds[];
   float* qs = lds;        // [dk]
   float* ps = lds + dk;   // [64]
@@ -107,9 +112,15 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
 
   float m = -INFINITY, l = 0.f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int c0 = (lo / 64) * 64; c0 <= pos; c0 += 64) {
+  // blocks of 64 keys aligned to absolute positions: first those that hold kept first positions in front of the
+  // window, then the window's; a block that holds both is visited once
+  const int keep = bp.window > 0 ? min(bp.keep_first, lo) : 0;      // keys below `keep` are seen although the window has passed them
+  const int win0 = (lo / 64) * 64;
+  const float inv_cap = bp.softcap > 0.f ? 1.0f / bp.softcap : 0.f;
+  for (int c0 = 0; c0 <= pos; c0 += 64) {
+    if (c0 >= keep && c0 < win0) { c0 = win0 - 64; continue; }
     const int key = c0 + lane;
-    const bool valid = key >= lo && key <= pos;
+    const bool valid = key <= pos && (key >= lo || key < keep);
     float s = -INFINITY;
     if (valid) {
       int page = bt[key / P];
@@ -118,6 +129,7 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
       float dot = 0.f;
       for (int j = 0; j < dk; j++) dot = fmaf(qs[j], load_f32(kp + j), dot);
       s = dot * qscale - slope * (float)(pos - key);
+      if (bp.softcap > 0.f) s = bp.softcap * tanhf(s * inv_cap);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float alpha = expf(m - m_new);
@@ -128,8 +140,9 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
     __syncthreads();
     float blk[4] = {0.f, 0.f, 0.f, 0.f};
     const int kend = min(64, pos - c0 + 1);
-    for (int kk = max(0, lo - c0); kk < kend; kk++) {
+    for (int kk = 0; kk < kend; kk++) {
       const int kpos = c0 + kk;
+      if (kpos < lo && kpos >= keep) continue;
       int page = bt[kpos / P];
       page = min(max(page, 0), num_pages - 1);
       const T* vp = v_cache + ((size_t)page * nkv + g) * dv * P + kpos % P;
@@ -148,7 +161,10 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int dim = lane + 64 * i;
-    if (dim < dv) store_f32(o + dim, acc[i] / l);
+    if (dim >= dv) continue;
+    float v = acc[i] / l;
+    if (gate) v *= 1.0f / (1.0f + expf(-load_f32(gate + (size_t)t * gate_stride + (size_t)h * dv + dim)));
+    store_f32(o + dim, v);
   }
 }
 
@@ -156,6 +172,7 @@ extern "C" int pico_attn_bias_plain(const void* q, int q_stride, int dtype, cons
                                     const int* block_table, int max_pages, const int* positions, const int* token_seq,
                                     void* out, int T, int nq, int nkv, int dk, int dv, int P, int window, float scale,
                                     float temp_coef, int temp_every, float slope_span, int num_pages,
+                                    float softcap, int keep_first, const void* gate, int gate_stride,
                                     hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && dk > 0 && dv > 0 && P > 0 && max_pages > 0 && num_pages > 0,
                "pico_attn_bias_plain: bad sizes");
@@ -164,18 +181,20 @@ extern "C" int pico_attn_bias_plain(const void* q, int q_stride, int dtype, cons
   PICO_REQUIRE(nq <= 65535, "pico_attn_bias_plain: too many heads");
   PICO_REQUIRE(q_stride >= nq * dk, "pico_attn_bias_plain: query row stride too small");
   PICO_REQUIRE(window >= 0 && temp_every >= 0 && slope_span >= 0.f, "pico_attn_bias_plain: window, interval and span must not be negative");
+  PICO_REQUIRE(softcap >= 0.f && keep_first >= 0, "pico_attn_bias_plain: cap and kept first positions must not be negative");
+  PICO_REQUIRE(gate == nullptr || gate_stride >= nq * dv, "pico_attn_bias_plain: gate row stride too small");
   if (T == 0) return 0;
-  const BiasParams bp{scale, temp_coef, slope_span, temp_every, window};
+  const BiasParams bp{scale, temp_coef, slope_span, temp_every, window, softcap, keep_first};
   dim3 grid(T, nq);
   const size_t lds = (size_t)(dk + 64) * sizeof(float);
   if (dtype == PICO_DTYPE_F32)
     attn_bias_plain_kernel<float><<<grid, 64, lds, stream>>>(
         (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, block_table, max_pages, positions,
-        token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages);
+        token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages, (const float*)gate, gate_stride);
   else if (dtype == PICO_DTYPE_BF16)
     attn_bias_plain_kernel<bf16_t><<<grid, 64, lds, stream>>>(
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, positions,
-        token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages);
+        token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages, (const bf16_t*)gate, gate_stride);
   else
     PICO_REQUIRE(false, "pico_attn_bias_plain: unknown dtype %d", dtype);
   PICO_LAUNCH_CHECK();

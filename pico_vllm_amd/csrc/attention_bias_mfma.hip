@@ -47,7 +47,15 @@ struct BiasArgs {
   int chunks, ncols;
   float* parts_o;
   float* parts_ml;
+  // scores <- softcap tanh(scores / softcap) (0: none); with a window, keys below keep_first are seen at any distance;
+  // gate (or null): the output is multiplied element by element with sigmoid(gate[t][head * DV + d])
+  float softcap;
+  int keep_first;
+  const bf16_t* gate;
+  int gate_stride;
 };
+
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
 template <bool SPLIT>
 __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
@@ -85,6 +93,8 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
   const int hi = p0 + ntok;                             // keys below hi are read
   const int lo = a.window > 0 ? max(0, p0 - a.window + 1) : 0;
   const int my_lo = a.window > 0 ? max(0, my_pos - a.window + 1) : 0;
+  const int keep = a.window > 0 ? a.keep_first : 0;     // keys below are seen although a window has passed them
+  const float inv_cap = a.softcap > 0.f ? 1.0f / a.softcap : 0.f;
   const int* bt = a.block_table + (size_t)b * a.max_pages;
   float qscale = a.scale, slope = 0.f;
   if (a.temp_every > 0) qscale *= 1.0f + a.temp_coef * logf((float)((my_pos + 1) / a.temp_every + 1));
@@ -114,11 +124,18 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
     begin += (int)blockIdx.z * piece;
     end = min(hi, begin + piece);
   }
+  // kept first keys in front of the window's first tile: tiles of their own, taken by the first piece (those inside
+  // the window's tiles are let through by the mask below)
+  const int sink_end = min(keep, lo & ~31);
+  const bool sinks = sink_end > 0 && (!SPLIT || blockIdx.z == 0);
   const int first = begin + (SPLIT ? 32 * wave : 0);
-  if (ntok > 0 && first < end) {
+  if (ntok > 0 && (first < end || sinks)) {
     const int last_key = hi - 1, last_group = last_key / 8 * 8;
     const int row_key = 8 * (col >> 2) + (col & 3);     // key of this lane's row in tile 0; tile 1: 4 more
-    for (int key0 = first; key0 < end; key0 += stride) {
+    int key0 = sinks ? (SPLIT ? 32 * wave : 0) : first;
+    bool in_sinks = sinks;
+    if (in_sinks && key0 >= sink_end) { in_sinks = false; key0 = first; }
+    while (in_sinks || key0 < end) {
       uint4 kr[2][KS];
       uint4 vr[DT];
       // positions beyond the range are clamped to its last key (group of 8, which lies in one page as pages hold at
@@ -150,7 +167,8 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
       for (int r = 0; r < 8; r++) {
         const int key = key0 + 8 * kq + r;
         float v = (r < 4 ? s0[r & 3] : s1[r & 3]) * qscale - slope * (float)(my_pos - key);
-        if (key > my_pos || key < my_lo) v = -INFINITY;
+        if (a.softcap > 0.f) v = a.softcap * tanhf(v * inv_cap);
+        if (key > my_pos || (key < my_lo && key >= keep)) v = -INFINITY;
         sv[r] = v;
         mx = fmaxf(mx, v);
       }
@@ -173,19 +191,21 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
                                                                pack2_bf16(sv[4], sv[5]), pack2_bf16(sv[6], sv[7])));
       if (key0 + 32 > hi || key0 < lo) {
         // values of keys outside the range hold whatever the page held before: make them zero (0 * NaN is NaN)
-        const int left = hi - (key0 + 8 * kq);                  // this lane's eight keys exist below `left` ...
-        const int skip = lo - (key0 + 8 * kq);                  // ... and from `skip` on
-        uint32_t keep[4];
+        // this lane's eight keys: a key counts if it lies below hi and either inside the block's window or among
+        // the kept first ones
+        uint32_t live[4];
 #pragma unroll
-        for (int w = 0; w < 4; w++)
-          keep[w] = ((left >= 2 * w + 2 ? 0xffffffffu : left == 2 * w + 1 ? 0x0000ffffu : 0u) &
-                     (skip <= 2 * w ? 0xffffffffu : skip == 2 * w + 1 ? 0xffff0000u : 0u));
+        for (int w = 0; w < 4; w++) {
+          const int k0 = key0 + 8 * kq + 2 * w, k1 = k0 + 1;
+          const bool v0 = k0 < hi && (k0 >= lo || k0 < keep), v1 = k1 < hi && (k1 >= lo || k1 < keep);
+          live[w] = (v0 ? 0x0000ffffu : 0u) | (v1 ? 0xffff0000u : 0u);
+        }
 #pragma unroll
         for (int tt = 0; tt < DT; tt++) {
-          vr[tt].x &= keep[0];
-          vr[tt].y &= keep[1];
-          vr[tt].z &= keep[2];
-          vr[tt].w &= keep[3];
+          vr[tt].x &= live[0];
+          vr[tt].y &= live[1];
+          vr[tt].z &= live[2];
+          vr[tt].w &= live[3];
         }
       }
 #pragma unroll
@@ -193,6 +213,8 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
         o[tt] *= alpha;
         o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vr[tt]), pb, o[tt], 0, 0, 0);
       }
+      key0 += stride;
+      if (in_sinks && key0 >= sink_end) { in_sinks = false; key0 = first; }
     }
   }
   float a0 = 1.f, L = l, M_all = m;
@@ -241,11 +263,20 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
   }
   const float inv = 1.0f / L;
   bf16_t* orow = a.out + ((size_t)t * a.nq + head) * DV + 4 * kq;
+  const bf16_t* grow = a.gate ? a.gate + (size_t)t * a.gate_stride + (size_t)head * DV + 4 * kq : nullptr;
 #pragma unroll
   for (int tt = 0; tt < DT; tt++) {
+    float g0 = inv, g1 = inv, g2 = inv, g3 = inv;
+    if (grow) {
+      const uint2 gv = *reinterpret_cast<const uint2*>(grow + 16 * tt);
+      g0 *= sigmoid_f32(__uint_as_float(gv.x << 16));
+      g1 *= sigmoid_f32(__uint_as_float(gv.x & 0xffff0000u));
+      g2 *= sigmoid_f32(__uint_as_float(gv.y << 16));
+      g3 *= sigmoid_f32(__uint_as_float(gv.y & 0xffff0000u));
+    }
     uint2 w;
-    w.x = pack2_bf16(o[tt][0] * inv, o[tt][1] * inv);
-    w.y = pack2_bf16(o[tt][2] * inv, o[tt][3] * inv);
+    w.x = pack2_bf16(o[tt][0] * g0, o[tt][1] * g1);
+    w.y = pack2_bf16(o[tt][2] * g2, o[tt][3] * g3);
     *reinterpret_cast<uint2*>(orow + 16 * tt) = w;
   }
 }
@@ -253,7 +284,8 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
 #define MAX_PIECES 64
 // The pieces of a column's keys put together: out = sum_z o_z e^(m_z - M) / sum_z l_z e^(m_z - M), z in ascending order.
 __global__ __launch_bounds__(DV <= 64 ? 64 : DV <= 128 ? 128 : 256) void attn_bias_merge_kernel(
-    const float* __restrict__ parts_o, const float* __restrict__ parts_ml, int chunks, int ncols, bf16_t* __restrict__ out) {
+    const float* __restrict__ parts_o, const float* __restrict__ parts_ml, int chunks, int ncols, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ gate, int gate_stride, int nq) {
   // the pieces' maxima and sums once into LDS (one load a thread, all in flight together), then every thread its sum
   __shared__ float ms[MAX_PIECES], ws[MAX_PIECES];
   const int c = blockIdx.x, d = threadIdx.x;
@@ -273,7 +305,9 @@ __global__ __launch_bounds__(DV <= 64 ? 64 : DV <= 128 ? 128 : 256) void attn_bi
     L += ws[z] * w;
     acc += parts_o[((size_t)z * ncols + c) * DV + d] * w;
   }
-  out[(size_t)c * DV + d] = f32_to_bf16(acc / L);
+  float v = acc / L;
+  if (gate) v *= sigmoid_f32(bf16_to_f32(gate[(size_t)(c / nq) * gate_stride + (size_t)(c % nq) * DV + d]));
+  out[(size_t)c * DV + d] = f32_to_bf16(v);
 }
 
 // split != 0: one block of 16 columns a workgroup, its keys shared by the four waves; else four blocks a workgroup.
@@ -281,7 +315,7 @@ extern "C" int pico_attnb(const void* q, int q_stride, const void* k_cache, cons
                           int max_pages, const int* cu_seqlens, const int* positions, int num_seqs, int T, void* out,
                           int nq, int nkv, int dk, int dv, int P, int num_pages, float scale, int window, float temp_coef,
                           int temp_every, float slope_span, int split, int chunks, float* parts_o, float* parts_ml,
-                          hipStream_t stream) {
+                          float softcap, int keep_first, const void* gate, int gate_stride, hipStream_t stream) {
   PICO_REQUIRE(dk == DK && dv == DV, "pico_attnb: built for keys of %d and values of %d, asked for %d and %d", DK, DV, dk, dv);
   PICO_REQUIRE(T >= 0 && num_seqs > 0 && nq > 0 && nkv > 0 && nq % nkv == 0 && max_pages > 0 && num_pages > 0,
                "pico_attnb: bad sizes");
@@ -290,6 +324,9 @@ extern "C" int pico_attnb(const void* q, int q_stride, const void* k_cache, cons
   PICO_REQUIRE(nkv <= 65535 && window >= 0 && temp_every >= 0 && slope_span >= 0.f, "pico_attnb: bad constants");
   PICO_REQUIRE(chunks >= 1 && chunks <= MAX_PIECES && (chunks == 1 || (split && parts_o && parts_ml)),
                "pico_attnb: pieces of the keys go with one block a workgroup and need room for the parts");
+  PICO_REQUIRE(softcap >= 0.f && keep_first >= 0, "pico_attnb: cap and kept first positions must not be negative");
+  PICO_REQUIRE(gate == nullptr || (gate_stride >= nq * DV && gate_stride % 4 == 0 && (uintptr_t)gate % 8 == 0),
+               "pico_attnb: gate rows must be 8-byte aligned and hold all heads");
   if (T == 0) return 0;
   const int R = nq / nkv;
   const int tpb = R >= 16 ? 1 : 16 / R, hb = R > 16 ? (R + 15) / 16 : 1;
@@ -298,12 +335,13 @@ extern "C" int pico_attnb(const void* q, int q_stride, const void* k_cache, cons
   PICO_REQUIRE(tiles < (1ll << 30), "pico_attnb: too many blocks");
   BiasArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
              cu_seqlens, positions, (bf16_t*)out, num_seqs, nq, nkv, P, num_pages, window, temp_every, scale, temp_coef,
-             slope_span, chunks, T * nq, parts_o, parts_ml};
+             slope_span, chunks, T * nq, parts_o, parts_ml, softcap, keep_first, (const bf16_t*)gate, gate_stride};
   if (split) {
     attn_bias_kernel<true><<<dim3((unsigned)tiles, nkv, chunks), 256, 0, stream>>>(a);
     if (chunks > 1)
       attn_bias_merge_kernel<<<T * nq, DV <= 64 ? 64 : DV <= 128 ? 128 : 256, 0, stream>>>(parts_o, parts_ml, chunks, T * nq,
-                                                                                           (bf16_t*)out);
+                                                                                           (bf16_t*)out, (const bf16_t*)gate,
+                                                                                           gate_stride, nq);
   } else
     attn_bias_kernel<false><<<dim3((unsigned)((tiles + 3) / 4), nkv), 256, 0, stream>>>(a);
   PICO_LAUNCH_CHECK();

@@ -281,22 +281,23 @@ extern "C" int pico_swiglu(const void* gu, void* out, int dtype, int T, int I, h
 // Grid T; block 256 (one workgroup per token).
 // ---------------------------------------------------------------------------
 __global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
-                                  float2* __restrict__ cos_sin, int half) {
+                                  float2* __restrict__ cos_sin, int half, float magnitude) {
   const int t = blockIdx.x;
   const float pos = (float)positions[t];
   for (int j = threadIdx.x; j < half; j += blockDim.x) {
     float c, s;
     sincosf(pos * inv_freq[j], &s, &c);
-    cos_sin[(size_t)t * half + j] = make_float2(c, s);
+    cos_sin[(size_t)t * half + j] = make_float2(c * magnitude, s * magnitude);
   }
 }
 
+// magnitude: a factor on every cosine and sine (1: none; scaled frequencies come with one)
 extern "C" int pico_rope_table(const int* positions, const float* inv_freq, float* cos_sin, int T, int half,
-                               hipStream_t stream) {
+                               float magnitude, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && half >= 0, "pico_rope_table: bad sizes");
   PICO_REQUIRE((uintptr_t)cos_sin % 8 == 0, "pico_rope_table: the table must be 8-byte aligned");
   if (T == 0 || half == 0) return 0;
-  rope_table_kernel<<<T, 64, 0, stream>>>(positions, inv_freq, (float2*)cos_sin, half);
+  rope_table_kernel<<<T, 64, 0, stream>>>(positions, inv_freq, (float2*)cos_sin, half, magnitude);
   PICO_LAUNCH_CHECK();
   return 0;
 }

@@ -6,6 +6,11 @@
 //                        y = g * sigmoid(alpha g) * (u + 1), out = Wd_e y
 //   a token's output: sum over its experts of expert_e(w_e * x)     (the weight scales the expert's INPUT)
 //
+// A second family (MOE_MODE_SOFTMAX_SWIGLU): scores s = softmax(z) over all router outputs; the `top` largest of
+// s + correction are chosen; weights = the chosen s over their sum, times a constant; an expert is
+// Wd_e (silu(Wg_e x) * (Wu_e x)) and the weight scales its OUTPUT (here: y, in front of the linear Wd_e); router outputs
+// from E on stand for experts that hand their input on unchanged.
+//
 // Expert matrices are stacked: gate_up [E, 2 F, D] (an expert's gate rows, then its up rows), down [E, D, F].
 // This file holds the plain kernels (one wave per output element, any sizes, float32 or bfloat16 storage, every sum
 // in float32 and in an order that depends on the sizes alone); the matrix-core kernels for many rows stand behind them.
@@ -105,8 +110,29 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const T* __restrict__ x
 }
 
 // router logits into z [T, E], then the choice: two launches
+__global__ void moe_route_softmax_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int T,
+                                         int E, int top, float scale, int* __restrict__ experts,
+                                         float* __restrict__ weights);
+
+static int moe_router_impl(const void* x, int ldx, int dtype, const float* Wr, int T, int E, int D, int top, float* z,
+                           int* experts, float* weights, int softmax, const float* correction, float scale,
+                           hipStream_t stream);
+
 extern "C" int pico_moe_router(const void* x, int ldx, int dtype, const float* Wr, int T, int E, int D, int top,
                                float* z, int* experts, float* weights, hipStream_t stream) {
+  return moe_router_impl(x, ldx, dtype, Wr, T, E, D, top, z, experts, weights, 0, nullptr, 1.f, stream);
+}
+
+// router logits, then the choice by softmax scores plus correction (see moe_route_softmax_kernel)
+extern "C" int pico_moe_router_softmax(const void* x, int ldx, int dtype, const float* Wr, const float* correction, int T,
+                                       int E, int D, int top, float scale, float* z, int* experts, float* weights,
+                                       hipStream_t stream) {
+  return moe_router_impl(x, ldx, dtype, Wr, T, E, D, top, z, experts, weights, 1, correction, scale, stream);
+}
+
+static int moe_router_impl(const void* x, int ldx, int dtype, const float* Wr, int T, int E, int D, int top, float* z,
+                           int* experts, float* weights, int softmax, const float* correction, float scale,
+                           hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && E > 0 && D > 0 && ldx >= D && top > 0 && top <= E && top <= MOE_MAX_TOP,
                "pico_moe_router: %d of %d experts per token is outside what the kernel takes (at most %d)", top, E, MOE_MAX_TOP);
   PICO_REQUIRE(dtype == PICO_DTYPE_F32 || dtype == PICO_DTYPE_BF16, "pico_moe_router: unknown dtype %d", dtype);
@@ -119,7 +145,10 @@ extern "C" int pico_moe_router(const void* x, int ldx, int dtype, const float* W
   if (dtype == PICO_DTYPE_F32) { if (vec) LAUNCH(float, true); else LAUNCH(float, false); }
   else { if (vec) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
 #undef LAUNCH
-  moe_route_kernel<<<(T + 63) / 64, 64, 0, stream>>>(z, T, E, top, experts, weights);
+  if (softmax)
+    moe_route_softmax_kernel<<<(T + 63) / 64, 64, 0, stream>>>(z, correction, T, E, top, scale, experts, weights);
+  else
+    moe_route_kernel<<<(T + 63) / 64, 64, 0, stream>>>(z, T, E, top, experts, weights);
   PICO_LAUNCH_CHECK();
   return 0;
 }
@@ -134,10 +163,98 @@ extern "C" int pico_moe_route(const float* logits, int T, int E, int top, int* e
   return 0;
 }
 
-__device__ __forceinline__ float expert_act(float g, float u, float limit, float alpha) {
+#define MOE_MODE_CLIPPED 0
+#define MOE_MODE_SOFTMAX_SWIGLU 1
+
+// mode 0: the clipped activation, the row's weight w already in the input; mode 1: w silu(g) u
+__device__ __forceinline__ float expert_act(float g, float u, float limit, float alpha, int mode, float w) {
+  if (mode == MOE_MODE_SOFTMAX_SWIGLU) return w * (g / (1.0f + expf(-g))) * u;
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+}
+
+// ---------------------------------------------------------------------------
+// Choice by softmax scores with a correction: one thread per token.  z [T, E] float32 router logits (E counts every
+// router output); correction [E] or null.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void moe_route_softmax_kernel(const float* __restrict__ logits,
+                                                               const float* __restrict__ correction, int T, int E, int top,
+                                                               float scale, int* __restrict__ experts,
+                                                               float* __restrict__ weights) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* z = logits + (size_t)t * E;
+  float mx = z[0];
+  for (int e = 1; e < E; e++) mx = fmaxf(mx, z[e]);
+  float den = 0.f;
+  for (int e = 0; e < E; e++) den += expf(z[e] - mx);
+  const float inv = 1.0f / den;
+  int chosen[MOE_MAX_TOP];
+  float score[MOE_MAX_TOP];
+  float total = 0.f;
+  for (int k = 0; k < top; k++) {
+    int best = -1;
+    float bc = 0.f, bs = 0.f;
+    for (int e = 0; e < E; e++) {
+      bool taken = false;
+      for (int j = 0; j < k; j++) taken |= chosen[j] == e;
+      if (taken) continue;
+      const float sc = expf(z[e] - mx) * inv;
+      const float c = sc + (correction ? correction[e] : 0.f);
+      if (best < 0 || c > bc) { best = e; bc = c; bs = sc; }
+    }
+    chosen[k] = best;
+    score[k] = bs;
+    total += bs;
+  }
+  const float f = scale / (total + 1e-20f);
+  for (int k = 0; k < top; k++) {
+    experts[(size_t)t * top + k] = chosen[k];
+    weights[(size_t)t * top + k] = score[k] * f;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Router outputs from E on are experts that hand their input on: for every (token, slot) with such an expert,
+// stacked: out[slot][t][:] = w h[t][:] (the slab rows that no expert's product writes); else out[t][:] += w h[t][:].
+// grid (T).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void moe_identity_kernel(const T* __restrict__ h, int ldh, const int* __restrict__ experts,
+                                                           const float* __restrict__ weights, float* __restrict__ out,
+                                                           int Tn, int top, int E, int D, int stacked) {
+  const int t = blockIdx.x;
+  const T* x = h + (size_t)t * ldh;
+  if (stacked) {
+    for (int k = 0; k < top; k++) {
+      if (experts[(size_t)t * top + k] < E) continue;
+      const float w = weights[(size_t)t * top + k];
+      float* o = out + ((size_t)k * Tn + t) * D;
+      for (int j = threadIdx.x; j < D; j += blockDim.x) o[j] = w * load_f32(x + j);
+    }
+    return;
+  }
+  float w = 0.f;
+  for (int k = 0; k < top; k++)
+    if (experts[(size_t)t * top + k] >= E) w += weights[(size_t)t * top + k];
+  if (w == 0.f) return;
+  float* o = out + (size_t)t * D;
+  for (int j = threadIdx.x; j < D; j += blockDim.x) o[j] = fmaf(w, load_f32(x + j), o[j]);
+}
+
+extern "C" int pico_moe_identity(const void* h, int ldh, int dtype, const int* experts, const float* weights, float* out,
+                                 int T, int top, int E, int D, int stacked, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && top > 0 && E >= 0 && D > 0 && ldh >= D, "pico_moe_identity: bad sizes");
+  if (T == 0) return 0;
+  if (dtype == PICO_DTYPE_F32)
+    moe_identity_kernel<float><<<T, 256, 0, stream>>>((const float*)h, ldh, experts, weights, out, T, top, E, D, stacked);
+  else if (dtype == PICO_DTYPE_BF16)
+    moe_identity_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)h, ldh, experts, weights, out, T, top, E, D, stacked);
+  else
+    PICO_REQUIRE(false, "pico_moe_identity: unknown dtype %d", dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
 }
 
 // the input of an expert: the token's row times its weight, rounded to the storage type as a product's operand is
@@ -155,11 +272,12 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_up_plain_kernel(const T* __restrict__ h, int ldh, const T* __restrict__ gate_up,
                                                            const int* __restrict__ experts, const float* __restrict__ weights,
                                                            T* __restrict__ y, int top, int E, int F, int D, float limit,
-                                                           float alpha) {
+                                                           float alpha, int mode) {
   const int r = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int e = experts[r];
   if (e < 0 || e >= E) return;
-  const float w = weights[r];
+  const float wr = weights[r];
+  const float w = mode == MOE_MODE_SOFTMAX_SWIGLU ? 1.f : wr;
   const T* x = h + (size_t)(r / top) * ldh;
   const T* We = gate_up + (size_t)e * 2 * F * D;
   for (int i = 0; i < 4; i++) {
@@ -169,13 +287,13 @@ __global__ __launch_bounds__(256) void moe_up_plain_kernel(const T* __restrict__
     const T* wu = We + (size_t)(F + f) * D;
     float g = 0.f, u = 0.f;
     for (int j = lane; j < D; j += 64) {
-      const float xv = scaled_input<T>(x + j, w);
+      const float xv = mode == MOE_MODE_SOFTMAX_SWIGLU ? load_f32(x + j) : scaled_input<T>(x + j, w);
       g = fmaf(load_f32(wg + j), xv, g);
       u = fmaf(load_f32(wu + j), xv, u);
     }
     g = wave_sum(g);
     u = wave_sum(u);
-    if (lane == 0) store_f32(y + (size_t)r * F + f, expert_act(g, u, limit, alpha));
+    if (lane == 0) store_f32(y + (size_t)r * F + f, expert_act(g, u, limit, alpha, mode, wr));
   }
 }
 
@@ -207,18 +325,19 @@ __global__ __launch_bounds__(256) void moe_down_plain_kernel(const T* __restrict
 
 extern "C" int pico_moe_experts_plain(const void* h, int ldh, int dtype, const void* gate_up, const void* down,
                                       const int* experts, const float* weights, void* y, float* out, int T, int top,
-                                      int E, int F, int D, float limit, float alpha, hipStream_t stream) {
+                                      int E, int F, int D, float limit, float alpha, int mode, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && top > 0 && E > 0 && F > 0 && D > 0 && ldh >= D, "pico_moe_experts_plain: bad sizes");
+  PICO_REQUIRE(mode == MOE_MODE_CLIPPED || mode == MOE_MODE_SOFTMAX_SWIGLU, "pico_moe_experts_plain: unknown mode %d", mode);
   if (T == 0) return 0;
   const dim3 g1(T * top, (F + 15) / 16), g2(T, (D + 15) / 16);
   PICO_REQUIRE(g1.y <= 65535 && g2.y <= 65535, "pico_moe_experts_plain: sizes beyond the grid");
   if (dtype == PICO_DTYPE_F32) {
     moe_up_plain_kernel<float><<<g1, 256, 0, stream>>>((const float*)h, ldh, (const float*)gate_up, experts, weights,
-                                                       (float*)y, top, E, F, D, limit, alpha);
+                                                       (float*)y, top, E, F, D, limit, alpha, mode);
     moe_down_plain_kernel<float><<<g2, 256, 0, stream>>>((const float*)y, (const float*)down, experts, out, top, E, F, D);
   } else if (dtype == PICO_DTYPE_BF16) {
     moe_up_plain_kernel<bf16_t><<<g1, 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)gate_up, experts, weights,
-                                                        (bf16_t*)y, top, E, F, D, limit, alpha);
+                                                        (bf16_t*)y, top, E, F, D, limit, alpha, mode);
     moe_down_plain_kernel<bf16_t><<<g2, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)down, experts, out, top, E, F, D);
   } else {
     PICO_REQUIRE(false, "pico_moe_experts_plain: unknown dtype %d", dtype);

@@ -20,7 +20,10 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define MOE_BK 64          // k of one stage
 #define MOE_LD 72          // LDS row stride in bfloat16: 144 bytes, a multiple of 16 that spreads rows over the banks
 
-__device__ __forceinline__ float moe_act(float g, float u, float limit, float alpha) {
+// mode 0: the clipped activation, the row's weight w already in the input; mode 1: w silu(g) u (the weight on the
+// expert's output, taken in front of the linear second product)
+__device__ __forceinline__ float moe_act(float g, float u, float limit, float alpha, int mode, float w) {
+  if (mode == 1) return w * (g / (1.0f + expf(-g))) * u;
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
@@ -75,19 +78,21 @@ __global__ __launch_bounds__(256) void moe_up_rows_kernel(const bf16_t* __restri
                                                           const bf16_t* __restrict__ gate_up,
                                                           const int* __restrict__ experts, const float* __restrict__ weights,
                                                           bf16_t* __restrict__ y, int top, int E, int F, int D, float limit,
-                                                          float alpha) {
+                                                          float alpha, int mode) {
   const int r = blockIdx.x, sub = threadIdx.x & 15;
   const int f = blockIdx.y * 16 + (threadIdx.x >> 4);
   const int e = experts[r];
   if (e < 0 || e >= E || f >= F) return;
-  const float w = weights[r];
+  const float wr = weights[r];
+  const float w = mode == 1 ? 1.f : wr;
   const bf16_t* x = h + (size_t)(r / top) * ldh;
   const bf16_t* wg = gate_up + ((size_t)e * 2 * F + f) * D;
   const bf16_t* wu = wg + (size_t)F * D;
   float g = 0.f, u = 0.f;
 #pragma unroll 2
   for (int k = sub * 8; k < D; k += 128) {
-    const uint4 xv = scale8(*reinterpret_cast<const uint4*>(x + k), w);
+    const uint4 x8 = *reinterpret_cast<const uint4*>(x + k);
+    const uint4 xv = mode == 1 ? x8 : scale8(x8, w);
     const uint4 gv = *reinterpret_cast<const uint4*>(wg + k);
     const uint4 uv = *reinterpret_cast<const uint4*>(wu + k);
     float xf[8];
@@ -97,7 +102,7 @@ __global__ __launch_bounds__(256) void moe_up_rows_kernel(const bf16_t* __restri
   }
   g = row16_sum(g);
   u = row16_sum(u);
-  if (sub == 0) y[(size_t)r * F + f] = f32_to_bf16(moe_act(g, u, limit, alpha));
+  if (sub == 0) y[(size_t)r * F + f] = f32_to_bf16(moe_act(g, u, limit, alpha, mode, wr));
 }
 
 // ---------------------------------------------------------------------------
@@ -130,8 +135,9 @@ __global__ __launch_bounds__(256) void moe_down_rows_kernel(const bf16_t* __rest
 
 extern "C" int pico_moe_experts_rows(const void* h, int ldh, const void* gate_up, const void* down, const int* experts,
                                      const float* weights, void* y, float* out, int T, int top, int E, int F, int D,
-                                     float limit, float alpha, hipStream_t stream) {
+                                     float limit, float alpha, int mode, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && top > 0 && E > 0 && F > 0 && D > 0 && ldh >= D, "pico_moe_experts_rows: bad sizes");
+  PICO_REQUIRE(mode == 0 || mode == 1, "pico_moe_experts_rows: unknown mode %d", mode);
   PICO_REQUIRE(F % 8 == 0 && D % 8 == 0 && ldh % 8 == 0, "pico_moe_experts_rows: sizes must be multiples of 8");
   PICO_REQUIRE(((uintptr_t)h | (uintptr_t)gate_up | (uintptr_t)down | (uintptr_t)y) % 16 == 0,
                "pico_moe_experts_rows: operands must start on 16 bytes");
@@ -139,7 +145,7 @@ extern "C" int pico_moe_experts_rows(const void* h, int ldh, const void* gate_up
   const dim3 g1(T * top, (F + 15) / 16), g2(T, (D + 15) / 16);
   PICO_REQUIRE(g1.y <= 65535 && g2.y <= 65535, "pico_moe_experts_rows: sizes beyond the grid");
   moe_up_rows_kernel<<<g1, 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)gate_up, experts, weights, (bf16_t*)y,
-                                             top, E, F, D, limit, alpha);
+                                             top, E, F, D, limit, alpha, mode);
   moe_down_rows_kernel<<<g2, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)down, experts, out, top, E, F, D);
   PICO_LAUNCH_CHECK();
   return 0;
@@ -213,7 +219,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
                                                           const int* __restrict__ tile_expert,
                                                           const float* __restrict__ weights, bf16_t* __restrict__ y,
                                                           float* __restrict__ out, int T, int top, int F, int D,
-                                                          float limit, float alpha, int ntile, int ncol) {
+                                                          float limit, float alpha, int ntile, int ncol, int mode) {
   __shared__ __attribute__((aligned(16))) bf16_t As[MOE_BM * MOE_LD];
   __shared__ __attribute__((aligned(16))) bf16_t Bs[MOE_BN * MOE_LD];
   __shared__ int rows[MOE_BM];
@@ -247,7 +253,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
       const int r = sorted[(size_t)tile * MOE_BM + m];                                    \
       A_OK = r >= 0;                                                                      \
       A_SRC = A + (size_t)(A_OK ? r / top : 0) * lda + sk;                                \
-      A_W = A_OK ? weights[r] : 0.f;                                                      \
+      A_W = A_OK ? (mode == 1 ? 1.f : weights[r]) : 0.f;                                  \
       const int f = c0 + (m & 63);                                                        \
       B_OK = f < F;                                                                       \
       B_SRC = W + ((size_t)e * erows + (B_OK ? (m >> 6) * F + f : 0)) * K + sk;           \
@@ -295,10 +301,11 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
       bf16_t* as = As + srow * MOE_LD + sk;
       bf16_t* bs = Bs + srow * MOE_LD + sk;
       const bool k_in = k0 + sk < K;
-      *reinterpret_cast<uint4*>(as) = keep8(UP ? scale8(ra0, a_w0) : ra0, a_ok0 && k_in);
-      *reinterpret_cast<uint4*>(as + 32 * MOE_LD) = keep8(UP ? scale8(ra1, a_w1) : ra1, a_ok1 && k_in);
-      *reinterpret_cast<uint4*>(as + 64 * MOE_LD) = keep8(UP ? scale8(ra2, a_w2) : ra2, a_ok2 && k_in);
-      *reinterpret_cast<uint4*>(as + 96 * MOE_LD) = keep8(UP ? scale8(ra3, a_w3) : ra3, a_ok3 && k_in);
+      const bool scaled = UP && mode != 1;        // mode 1 puts the weight on the activation instead
+      *reinterpret_cast<uint4*>(as) = keep8(scaled ? scale8(ra0, a_w0) : ra0, a_ok0 && k_in);
+      *reinterpret_cast<uint4*>(as + 32 * MOE_LD) = keep8(scaled ? scale8(ra1, a_w1) : ra1, a_ok1 && k_in);
+      *reinterpret_cast<uint4*>(as + 64 * MOE_LD) = keep8(scaled ? scale8(ra2, a_w2) : ra2, a_ok2 && k_in);
+      *reinterpret_cast<uint4*>(as + 96 * MOE_LD) = keep8(scaled ? scale8(ra3, a_w3) : ra3, a_ok3 && k_in);
       *reinterpret_cast<uint4*>(bs) = keep8(rb0, b_ok0 && k_in);
       *reinterpret_cast<uint4*>(bs + 32 * MOE_LD) = keep8(rb1, b_ok1 && k_in);
       *reinterpret_cast<uint4*>(bs + 64 * MOE_LD) = keep8(rb2, b_ok2 && k_in);
@@ -325,7 +332,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
     const int m = wm * 64 + 32 * (i) + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);                                     \
     if (UP) {                                                                                                        \
       const int f = c0 + wn * 32 + (lane & 31);                                                                      \
-      if (f < F) y[((size_t)tile * MOE_BM + m) * F + f] = f32_to_bf16(moe_act(ACC0[r], ACC1[r], limit, alpha));      \
+      const float wrow = (mode == 1 && rows[m] >= 0) ? weights[rows[m]] : 0.f;                                       \
+      if (f < F) y[((size_t)tile * MOE_BM + m) * F + f] = f32_to_bf16(moe_act(ACC0[r], ACC1[r], limit, alpha, mode, wrow)); \
     } else {                                                                                                         \
       const int row = rows[m];                                                                                       \
       if (row < 0) continue;                                                                                         \
@@ -345,7 +353,8 @@ extern "C" int pico_moe_tile_rows() { return MOE_BM; }
 extern "C" int pico_moe_experts_grouped(const void* h, int ldh, const void* gate_up, const void* down, const int* experts,
                                         const float* weights, int* sorted, int* tile_expert, int tiles_cap, void* y,
                                         float* out, int T, int top, int E, int F, int D, float limit, float alpha,
-                                        hipStream_t stream) {
+                                        int mode, hipStream_t stream) {
+  PICO_REQUIRE(mode == 0 || mode == 1, "pico_moe_experts_grouped: unknown mode %d", mode);
   PICO_REQUIRE(T >= 0 && top > 0 && E > 0 && F > 0 && D > 0 && ldh >= D, "pico_moe_experts_grouped: bad sizes");
   PICO_REQUIRE(E <= MOE_SORT_MAX_E, "pico_moe_experts_grouped: at most %d experts", MOE_SORT_MAX_E);
   PICO_REQUIRE(F % 8 == 0 && D % 8 == 0 && ldh % 8 == 0, "pico_moe_experts_grouped: sizes must be multiples of 8");
@@ -362,10 +371,10 @@ extern "C" int pico_moe_experts_grouped(const void* h, int ldh, const void* gate
   moe_sort_kernel<<<E, MOE_SORT_THREADS, 0, stream>>>(experts, (int)R, E, tiles_cap, sorted, tile_expert);
   moe_grouped_kernel<true><<<(unsigned)(slots * ncol1), 256, 0, stream>>>(
       (const bf16_t*)h, ldh, (const bf16_t*)gate_up, sorted, tile_expert, weights, (bf16_t*)y, nullptr, T, top, F, D, limit,
-      alpha, tiles_cap, (int)ncol1);
+      alpha, tiles_cap, (int)ncol1, mode);
   moe_grouped_kernel<false><<<(unsigned)(slots * ncol2), 256, 0, stream>>>(
       (const bf16_t*)y, F, (const bf16_t*)down, sorted, tile_expert, nullptr, nullptr, out, T, top, F, D, limit, alpha,
-      tiles_cap, (int)ncol2);
+      tiles_cap, (int)ncol2, mode);
   PICO_LAUNCH_CHECK();
   return 0;
 }

@@ -24,7 +24,7 @@ import numpy as np
 
 
 class TraceReplayer:
-    def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, max_live: int = 8,
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, max_live: int = 4,
                  device: str = "cuda:0"):
         import torch
         from ..parts.model import load_model

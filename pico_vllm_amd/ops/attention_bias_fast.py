@@ -23,9 +23,11 @@ def supported(key_dim: int, value_dim: int) -> bool:
 
 class FastBiasAttention:
     def __init__(self, nq: int, nkv: int, key_dim: int, value_dim: int, scale: float, window: int = 0,
-                 temp_coef: float = 0.0, temp_every: int = 0, slope_span: float = 0.0):
+                 temp_coef: float = 0.0, temp_every: int = 0, slope_span: float = 0.0, softcap: float = 0.0,
+                 keep_first: int = 0, gated: bool = False):
         self.nq, self.nkv, self.dk, self.dv = nq, nkv, key_dim, value_dim
         self.scale, self.window, self.temp_coef, self.temp_every, self.slope_span = scale, window, temp_coef, temp_every, slope_span
+        self.softcap, self.keep_first, self.gated = float(softcap), int(keep_first), bool(gated)
         self.lib = library.attention_bias_library(key_dim, value_dim)
         if self.lib.pico_attnb_key_dim() != key_dim or self.lib.pico_attnb_value_dim() != value_dim:
             raise KernelError("attention library was built for other sizes")
@@ -33,7 +35,9 @@ class FastBiasAttention:
         # keys and values of one size in steps of 32: prompt steps go through the rotary attention's prompt kernel (keys
         # staged in LDS for 64 or 128 queries), which takes the columns' factors and the penalty into its scores
         self.tuned = None
-        if key_dim == value_dim and key_dim % 32 == 0 and attention_fast.supported(nq, nkv, key_dim, window):
+        # (that kernel knows no cap on the scores, no kept first positions and no gate)
+        if key_dim == value_dim and key_dim % 32 == 0 and attention_fast.supported(nq, nkv, key_dim, window) \
+                and not (self.softcap > 0 or (self.keep_first > 0 and window > 0) or self.gated):
             self.tuned = attention_fast.FastAttention(nq, nkv, key_dim, window)
 
     def split(self, num_tokens: int) -> bool:
@@ -73,8 +77,10 @@ class FastBiasAttention:
         return (bool(self.split(ctx.num_tokens)), self.chunks(ctx.num_tokens, ctx.num_seqs), self.prompt_shape(ctx))
 
     def run(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, positions, num_seqs: int,
-            split: Optional[bool] = None, out: Optional[torch.Tensor] = None, chunks: Optional[int] = None) -> torch.Tensor:
-        """q [T, >= nq * dk] bfloat16 (row stride free); any mixture of portions and single tokens; returns [T, nq * dv]."""
+            split: Optional[bool] = None, out: Optional[torch.Tensor] = None, chunks: Optional[int] = None,
+            gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """q [T, >= nq * dk] bfloat16 (row stride free); any mixture of portions and single tokens; returns [T, nq * dv].
+        ``gate`` [T, >= nq * dv] bfloat16 (8-byte aligned rows): the output is multiplied with sigmoid(gate)."""
         T = q.shape[0]
         pages, P = _check_cache2(k_cache, v_cache, self.nkv, self.dk, self.dv)
         if not q.is_cuda or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
@@ -89,6 +95,10 @@ class FastBiasAttention:
                 raise KernelError("sequence metadata must be contiguous int32")
         if P < 8 or P & (P - 1):
             raise KernelError("matrix-core attention wants pages of a power of two of at least 8 tokens")
+        if gate is not None and (not gate.is_cuda or gate.dtype != torch.bfloat16 or gate.dim() != 2 or gate.shape[0] != T
+                                 or gate.stride(1) != 1 or gate.shape[1] < self.nq * self.dv or (T > 1 and gate.stride(0) % 4)
+                                 or gate.data_ptr() % 8):
+            raise KernelError("the gate must be bfloat16 [T, >= nq*dv] with unit stride along the row and 8-byte aligned rows")
         if out is None:
             out = torch.empty(T, self.nq * self.dv, dtype=torch.bfloat16, device=q.device)
         if split is None:
@@ -105,10 +115,11 @@ class FastBiasAttention:
             _ptr(q), q.stride(0) if T > 1 else q.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
             _ptr(cu_seqlens), _ptr(positions), num_seqs, T, _ptr(out), self.nq, self.nkv, self.dk, self.dv, P, pages,
             c_float(self.scale), self.window, c_float(self.temp_coef), self.temp_every, c_float(self.slope_span),
-            1 if split else 0, chunks, _ptr(parts_o), _ptr(parts_ml), _stream()))
+            1 if split else 0, chunks, _ptr(parts_o), _ptr(parts_ml), c_float(self.softcap), self.keep_first, _ptr(gate),
+            0 if gate is None else (gate.stride(0) if T > 1 else gate.shape[1]), _stream()))
         return out
 
-    def __call__(self, qkv, cache, block_table, ctx):
+    def __call__(self, qkv, cache, block_table, ctx, gate=None):
         split, chunks, shape = self.plan(ctx)
         if shape and cache.k.numel() * cache.k.element_size() < (1 << 32):
             B = ctx.num_seqs
@@ -122,7 +133,7 @@ class FastBiasAttention:
                                       teams=shape, order=order, order_build=build,
                                       scored=(self.temp_coef, self.temp_every, self.slope_span))
         return self.run(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.positions, ctx.num_seqs,
-                        split=split, chunks=chunks)
+                        split=split, chunks=chunks, gate=gate)
 
 
 def choose(mixer) -> Optional[FastBiasAttention]:
@@ -130,4 +141,5 @@ def choose(mixer) -> Optional[FastBiasAttention]:
     if not supported(mixer.dk, mixer.dv):
         return None
     return FastBiasAttention(mixer.nq, mixer.nkv, mixer.dk, mixer.dv, mixer.scale, mixer.window, mixer.temp_coef,
-                             mixer.temp_every, mixer.slope_span)
+                             mixer.temp_every, mixer.slope_span, getattr(mixer, "softcap", 0.0),
+                             getattr(mixer, "keep_first", 0), getattr(mixer, "gated", False))

@@ -299,8 +299,8 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int)
     return pages, P
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
-    """cos and sin of position * inv_freq in float32: [T, len(inv_freq), 2].  Every layer of a step
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, magnitude: float = 1.0) -> torch.Tensor:
+    """cos and sin of position * inv_freq in float32, times ``magnitude``: [T, len(inv_freq), 2].  Every layer of a step
     rotates by the same angles, so a step computes them once."""
     _gpu(positions, inv_freq)
     T = positions.numel()
@@ -309,7 +309,8 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
         raise KernelError("inv_freq must be contiguous float32")
     out = torch.empty(T, inv_freq.numel(), 2, dtype=torch.float32, device=positions.device)
     lib = library.core()
-    _check(lib, lib.pico_rope_table(_ptr(positions), _ptr(inv_freq), _ptr(out), T, inv_freq.numel(), _stream()))
+    _check(lib, lib.pico_rope_table(_ptr(positions), _ptr(inv_freq), _ptr(out), T, inv_freq.numel(), c_float(magnitude),
+                                    _stream()))
     return out
 
 
@@ -601,10 +602,13 @@ def kv_mix_store(qkv: torch.Tensor, k_col: int, v_col: int, slots: torch.Tensor,
 def attn_bias_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                     positions: torch.Tensor, token_seq: torch.Tensor, nq: int, nkv: int, dk: int, dv: int, scale: float,
                     window: int = 0, temp_coef: float = 0.0, temp_every: int = 0, slope_span: float = 0.0,
-                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    out: Optional[torch.Tensor] = None, softcap: float = 0.0, keep_first: int = 0,
+                    gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention with a distance penalty slope_h (i - j), slope_h = 2^(-slope_span (h + 1) / nq), and the query
-    temperature 1 + temp_coef ln(floor((i + 1) / temp_every) + 1) on the scores.  q: [T, >= nq * dk]; returns [T, nq * dv]."""
-    _gpu(q, k_cache, v_cache, block_table, positions, token_seq)
+    temperature 1 + temp_coef ln(floor((i + 1) / temp_every) + 1) on the scores.  q: [T, >= nq * dk]; returns [T, nq * dv].
+    ``softcap`` > 0: scores <- softcap tanh(scores / softcap).  ``keep_first``: with a window, keys at positions below it
+    stay visible.  ``gate`` [T, >= nq * dv] (row stride free): the output is multiplied with sigmoid(gate)."""
+    _gpu(q, k_cache, v_cache, block_table, positions, token_seq, gate)
     T = q.shape[0]
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < nq * dk:
         raise KernelError("q must be [T, >= nq*dk] with unit stride along the row")
@@ -619,11 +623,105 @@ def attn_bias_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         out = torch.empty(T, nq * dv, dtype=q.dtype, device=q.device)
     elif out.shape != (T, nq * dv) or out.dtype != q.dtype or not out.is_contiguous():
         raise KernelError("attention: out has the wrong shape or dtype")
+    if gate is not None and (gate.dtype != q.dtype or gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[0] != T
+                             or gate.shape[1] < nq * dv):
+        raise KernelError(f"attention: the gate must be [T, >= {nq * dv}] of the activations' dtype")
     lib = library.core()
     _check(lib, lib.pico_attn_bias_plain(_ptr(q), q.stride(0) if T > 1 else q.shape[1], _dt(q), _ptr(k_cache), _ptr(v_cache),
                                          _ptr(block_table), block_table.shape[1], _ptr(positions), _ptr(token_seq), _ptr(out),
                                          T, nq, nkv, dk, dv, P, window, c_float(scale), c_float(temp_coef), temp_every,
-                                         c_float(slope_span), pages, _stream()))
+                                         c_float(slope_span), pages, c_float(softcap), keep_first, _ptr(gate),
+                                         0 if gate is None else (gate.stride(0) if T > 1 else gate.shape[1]), _stream()))
+    return out
+
+
+def rope_pairs_store(x: torch.Tensor, q_col: int, k_col: int, v_col: int, cos_sin: Optional[torch.Tensor], rotary_dim: int,
+                     slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                     nq: int, nkv: int, dk: int, dv: int) -> None:
+    """Turn neighbouring pairs (2i, 2i + 1) of the first ``rotary_dim`` entries of every query head (in place, columns
+    q_col ..) and key head (columns k_col ..) of ``x`` [T, columns] by the angles of ``cos_sin`` (``rope_table``), and
+    write keys and values (columns v_col ..) to ``slots`` of the cache.  Without a cache only the queries are turned."""
+    _gpu(x, cos_sin, slots, k_cache, v_cache)
+    T = x.shape[0]
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < q_col + nq * dk:
+        raise KernelError("rope_pairs_store: x must be [T, columns] with unit stride along the row and hold the queries")
+    pages = P = 0
+    if k_cache is not None:
+        pages, P = _check_cache2(k_cache, v_cache, nkv, dk, dv)
+        if k_cache.dtype != x.dtype:
+            raise KernelError("cache and activations differ in dtype")
+        if x.shape[1] < max(k_col + nkv * dk, v_col + nkv * dv):
+            raise KernelError("rope_pairs_store: the rows do not hold the keys and values")
+        _i32(slots, "slots", T)
+    if rotary_dim % 2 or not 0 <= rotary_dim <= dk:
+        raise KernelError(f"rope_pairs_store: {rotary_dim} rotated entries do not fit a head of {dk}")
+    _check_table(cos_sin, T, rotary_dim // 2)
+    lib = library.core()
+    _check(lib, lib.pico_rope_pairs_store(_ptr(x), _dt(x), x.stride(0) if T > 1 else x.shape[1], q_col, k_col, v_col,
+                                          _ptr(cos_sin) if rotary_dim else None, rotary_dim, _ptr(slots), _ptr(k_cache),
+                                          _ptr(v_cache), T, nq, nkv, dk, dv, P, pages, _stream()))
+
+
+def gla_decay(x: torch.Tensor, col: int, a2: torch.Tensor, bias: Optional[torch.Tensor], tau: float) -> torch.Tensor:
+    """float32 [T, C]: log(sigmoid(z)) / tau with z = x[:, col : col + R] a2^T + bias; a2 [C, R] of x's dtype, bias float32."""
+    _gpu(x, a2, bias)
+    T = x.shape[0]
+    C, R = a2.shape
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < col + R or a2.dtype != x.dtype or not a2.is_contiguous():
+        raise KernelError("gla_decay: x [T, >= col + R] with unit stride along the row and a2 [C, R] of the same dtype")
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (C,) or not bias.is_contiguous()):
+        raise KernelError(f"gla_decay: bias must be contiguous float32 [{C}]")
+    out = torch.empty(T, C, dtype=torch.float32, device=x.device)
+    lib = library.core()
+    xv = x[:, col:]
+    _check(lib, lib.pico_gla_decay(_ptr(xv), x.stride(0) if T > 1 else x.shape[1], _dt(x), _ptr(a2), _ptr(bias), c_float(tau),
+                                   _ptr(out), T, C, R, _stream()))
+    return out
+
+
+GLA_MAX_KEY_DIM = 256
+
+
+def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: torch.Tensor, cu_seqlens: torch.Tensor,
+             state_slots: torch.Tensor, state: torch.Tensor, num_seqs: int, heads: int, dk: int, dv: int,
+             qscale: float) -> torch.Tensor:
+    """The recurrence S <- diag(exp(log_decay_t)) S + k_t v_t^T, o_t = S^T q_t qscale, for every sequence of the step from
+    its state slot (``state`` float32 [slots, heads, dk, dv], updated in place).  Returns o float32 [T, heads * dv]."""
+    _gpu(x, log_decay, cu_seqlens, state_slots, state)
+    T = x.shape[0]
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < max(q_col + heads * dk, k_col + heads * dk, v_col + heads * dv):
+        raise KernelError("gla_scan: x must be [T, columns] with unit stride along the row and hold q, k and v")
+    if log_decay.dtype != torch.float32 or tuple(log_decay.shape) != (T, heads * dk) or not log_decay.is_contiguous():
+        raise KernelError(f"gla_scan: the decays' logarithms must be contiguous float32 [{T}, {heads * dk}]")
+    if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dk, dv) or not state.is_contiguous():
+        raise KernelError(f"gla_scan: the state must be contiguous float32 [slots, {heads}, {dk}, {dv}]")
+    if dk > GLA_MAX_KEY_DIM:
+        raise KernelError(f"gla_scan: at most {GLA_MAX_KEY_DIM} key channels a head")
+    _i32(cu_seqlens, "cu_seqlens", num_seqs + 1)
+    _i32(state_slots, "state_slots", num_seqs)
+    out = torch.empty(T, heads * dv, dtype=torch.float32, device=x.device)
+    lib = library.core()
+    _check(lib, lib.pico_gla_scan(_ptr(x), x.stride(0) if T > 1 else x.shape[1], _dt(x), q_col, k_col, v_col, _ptr(log_decay),
+                                  _ptr(cu_seqlens), _ptr(state_slots), _ptr(state), _ptr(out), num_seqs, T, heads, dk, dv,
+                                  c_float(qscale), state.shape[0], _stream()))
+    return out
+
+
+def gla_out(o: torch.Tensor, x: torch.Tensor, g_col: int, weight: torch.Tensor, eps: float, heads: int, dv: int) -> torch.Tensor:
+    """[T, heads * dv] of x's dtype: every head of ``o`` (float32) RMS-normed over its dv entries with ``weight`` [dv],
+    times silu of the gate (columns g_col .. of x)."""
+    _gpu(o, x, weight)
+    T = o.shape[0]
+    if o.dtype != torch.float32 or tuple(o.shape) != (T, heads * dv) or not o.is_contiguous():
+        raise KernelError(f"gla_out: o must be contiguous float32 [T, {heads * dv}]")
+    if x.dim() != 2 or x.shape[0] != T or x.stride(1) != 1 or x.shape[1] < g_col + heads * dv:
+        raise KernelError("gla_out: the rows do not hold the gate")
+    if weight.dtype != torch.float32 or weight.shape != (dv,) or not weight.is_contiguous():
+        raise KernelError(f"gla_out: the norm's weight must be contiguous float32 [{dv}]")
+    out = torch.empty(T, heads * dv, dtype=x.dtype, device=x.device)
+    lib = library.core()
+    _check(lib, lib.pico_gla_out(_ptr(o), _ptr(x[:, g_col:]), x.stride(0) if T > 1 else x.shape[1], _dt(x), _ptr(weight),
+                                 c_float(eps), _ptr(out), T, heads, dv, _stream()))
     return out
 
 
@@ -667,6 +765,52 @@ def moe_router(x: torch.Tensor, w_router: torch.Tensor, top: int):
     return experts, weights
 
 
+def moe_router_softmax(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int, scale: float):
+    """Router and choice by softmax scores: z = x w_router^T in float32, s = softmax(z) over all E router outputs; the
+    ``top`` largest of s + correction are chosen (the lowest index among equals); weights = the chosen s over their sum
+    (+ 1e-20) times ``scale``.  Returns (experts int32 [T, top], weights float32 [T, top])."""
+    _gpu(x, w_router, correction)
+    T, D = x.shape
+    E = w_router.shape[0]
+    if w_router.dtype != torch.float32 or w_router.dim() != 2 or w_router.shape[1] != D or not w_router.is_contiguous():
+        raise KernelError(f"moe_router_softmax: the router matrix must be contiguous float32 [outputs, {D}]")
+    if correction is not None and (correction.dtype != torch.float32 or correction.shape != (E,) or not correction.is_contiguous()):
+        raise KernelError(f"moe_router_softmax: the correction must be contiguous float32 [{E}]")
+    if x.stride(1) != 1:
+        raise KernelError("moe_router_softmax: activations must have unit stride along the row")
+    if not 1 <= top <= min(E, MOE_MAX_TOP):
+        raise KernelError(f"moe_router_softmax: {top} of {E} experts per token (at most {MOE_MAX_TOP})")
+    z = torch.empty(T, E, dtype=torch.float32, device=x.device)
+    experts = torch.empty(T, top, dtype=torch.int32, device=x.device)
+    weights = torch.empty(T, top, dtype=torch.float32, device=x.device)
+    lib = library.core()
+    _check(lib, lib.pico_moe_router_softmax(_ptr(x), x.stride(0) if T > 1 else D, _dt(x), _ptr(w_router), _ptr(correction),
+                                            T, E, D, top, c_float(scale), _ptr(z), _ptr(experts), _ptr(weights), _stream()))
+    return experts, weights
+
+
+def moe_identity(h: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, num_experts: int) -> torch.Tensor:
+    """Experts numbered from ``num_experts`` on hand their input on: ``out`` float32 [T, D] += sum of their weights
+    times h; or, for a stack [top, T, D] of slabs (one a slot), the slab rows of such slots = weight times h (no
+    expert's product writes them)."""
+    _gpu(h, experts, weights, out)
+    T, D = h.shape
+    top = experts.shape[1]
+    stacked = out.dim() == 3
+    if out.dtype != torch.float32 or not out.is_contiguous() or tuple(out.shape) != ((top, T, D) if stacked else (T, D)):
+        raise KernelError("moe_identity: out must be contiguous float32 [T, D] or [top, T, D]")
+    if experts.dtype != torch.int32 or weights.dtype != torch.float32 or experts.shape != weights.shape \
+            or experts.shape[0] != T or not experts.is_contiguous() or not weights.is_contiguous() or h.stride(1) != 1:
+        raise KernelError("moe_identity: experts int32 [T, top], weights float32 [T, top], rows with unit stride")
+    lib = library.core()
+    _check(lib, lib.pico_moe_identity(_ptr(h), h.stride(0) if T > 1 else D, _dt(h), _ptr(experts), _ptr(weights), _ptr(out),
+                                      T, top, num_experts, D, int(stacked), _stream()))
+    return out
+
+
+MOE_CLIPPED, MOE_SWIGLU = 0, 1      # the experts' activation: clipped with the weight on the input; silu(g) u, weight on the output
+
+
 def _check_experts(h, gate_up, down, experts, weights, who):
     T, D = h.shape
     if gate_up.dim() != 3 or down.dim() != 3 or gate_up.shape[1] % 2:
@@ -685,7 +829,7 @@ def _check_experts(h, gate_up, down, experts, weights, who):
 
 
 def moe_experts_plain(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, experts: torch.Tensor,
-                      weights: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+                      weights: torch.Tensor, limit: float, alpha: float, mode: int = MOE_CLIPPED) -> torch.Tensor:
     """float32 [T, D]: sum over a token's experts of down_e(act(gate_up_e (w h))), by the plain kernels."""
     _gpu(h, gate_up, down, experts, weights)
     T, D, E, F, top = _check_experts(h, gate_up, down, experts, weights, "moe_experts_plain")
@@ -694,7 +838,7 @@ def moe_experts_plain(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor
     lib = library.core()
     _check(lib, lib.pico_moe_experts_plain(_ptr(h), h.stride(0) if T > 1 else D, _dt(h), _ptr(gate_up), _ptr(down),
                                            _ptr(experts), _ptr(weights), _ptr(y), _ptr(out), T, top, E, F, D,
-                                           c_float(limit), c_float(alpha), _stream()))
+                                           c_float(limit), c_float(alpha), mode, _stream()))
     return out
 
 
@@ -716,7 +860,8 @@ def moe_grouped_rows(tokens: int, top: int) -> bool:
 
 
 def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, experts: torch.Tensor,
-                weights: torch.Tensor, limit: float, alpha: float, grouped: Optional[bool] = None) -> torch.Tensor:
+                weights: torch.Tensor, limit: float, alpha: float, grouped: Optional[bool] = None,
+                mode: int = MOE_CLIPPED) -> torch.Tensor:
     """The experts' outputs in bfloat16 storage: float32 [T, D] (few rows: each streams its expert's matrices), or a
     float32 stack [top, T, D] whose sum over the first index it is (many rows: sorted by expert on the device and
     multiplied on the matrix cores)."""
@@ -732,15 +877,17 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, expe
         y = torch.empty(T * top, F, dtype=h.dtype, device=h.device)
         out = torch.empty(T, D, dtype=torch.float32, device=h.device)
         _check(lib, lib.pico_moe_experts_rows(_ptr(h), ldh, _ptr(gate_up), _ptr(down), _ptr(experts), _ptr(weights),
-                                              _ptr(y), _ptr(out), T, top, E, F, D, c_float(limit), c_float(alpha), _stream()))
+                                              _ptr(y), _ptr(out), T, top, E, F, D, c_float(limit), c_float(alpha), mode, _stream()))
         return out
     bm = lib.pico_moe_tile_rows()
     tiles = (T * top + E * (bm - 1)) // bm
     sorted_rows = torch.empty(tiles * bm, dtype=torch.int32, device=h.device)
     tile_expert = torch.empty(tiles, dtype=torch.int32, device=h.device)
     y = torch.empty(tiles * bm, F, dtype=h.dtype, device=h.device)
-    out = torch.empty(top, T, D, dtype=torch.float32, device=h.device)
+    # a slot whose expert has no matrices (a number from E on) is written by no product: with one slot a token the
+    # caller adds into the rows, which then start from zero; with several, ``moe_identity`` fills the slabs' rows
+    out = (torch.zeros if top == 1 else torch.empty)(top, T, D, dtype=torch.float32, device=h.device)
     _check(lib, lib.pico_moe_experts_grouped(_ptr(h), ldh, _ptr(gate_up), _ptr(down), _ptr(experts), _ptr(weights),
                                              _ptr(sorted_rows), _ptr(tile_expert), tiles, _ptr(y), _ptr(out), T, top, E, F,
-                                             D, c_float(limit), c_float(alpha), _stream()))
+                                             D, c_float(limit), c_float(alpha), mode, _stream()))
     return out[0] if top == 1 else out

@@ -66,3 +66,34 @@ class ParallelBlock(Block):
         for delta in (a if a.dim() == 3 else (a,)):            # a stack of partial sums: each in turn
             kernels.residual_add(resid, delta)
         return resid, f
+
+
+@register_part("block", "parallel_two_norms")
+class ParallelTwoNormBlock(Block):
+    """x += mixer(norm1(x)) + ff(norm2(x)): both sublayers read the same x, each through a norm of its own.  The sums
+    are float32.  A delta that is still pending joins the stream in the first norm's launch; the second norm then reads
+    the summed stream.  The mixer's output joins the stream at once, the feed-forward's last delta is handed on as
+    ``pending`` (a feed-forward may return a list of deltas: all but the last are added here).  A layer without a
+    feed-forward names the part "none" in that slot."""
+    slot_categories = {"norm1": "norm", "mixer": "mixer", "norm2": "norm", "ff": "feed_forward"}
+    graph_safe_prompts = True
+
+    @staticmethod
+    def _add(resid, delta):
+        for d in (delta if delta.dim() == 3 else (delta,)):    # a stack of partial sums: each in turn
+            kernels.residual_add(resid, d)
+
+    def forward(self, resid, pending, ctx, cache):
+        p = self.parts
+        h1 = p["norm1"].add_norm(resid, pending)
+        h2 = p["norm2"].add_norm(resid, None)
+        a = p["mixer"].forward(h1, ctx, cache)
+        f = p["ff"].forward(h2, ctx)
+        if f is None:
+            return resid, a
+        self._add(resid, a)
+        if isinstance(f, (list, tuple)):
+            for d in f[:-1]:
+                self._add(resid, d)
+            f = f[-1]
+        return resid, f

@@ -21,21 +21,24 @@ class SwiGLUMLP(FeedForward):
     takes_deferred_norm = True      # Linear.swiglu runs or fuses it
     graph_safe_prompts = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int, act_dtype: torch.dtype = torch.bfloat16):
+    def __init__(self, hidden_size: int, intermediate_size: int, act_dtype: torch.dtype = torch.bfloat16,
+                 names: tuple = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+        # names: the three matrices' names behind the part's prefix (gate, up, down)
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.names = tuple(names)
         self.gate_up: Optional[Linear] = None
         self.down: Optional[Linear] = None
 
     def param_specs(self) -> List[ParamSpec]:
         H, I = self.hidden_size, self.intermediate_size
-        return [ParamSpec("gate_proj.weight", (I, H)), ParamSpec("up_proj.weight", (I, H)),
-                ParamSpec("down_proj.weight", (H, I))]
+        g, u, d = self.names
+        return [ParamSpec(g, (I, H)), ParamSpec(u, (I, H)), ParamSpec(d, (H, I))]
 
     def load(self, tensors: Dict[str, torch.Tensor], device, dtype) -> None:
-        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        g, u = tensors[self.names[0]], tensors[self.names[1]]
         wdt = torch.float32 if torch.float32 in (g.dtype, u.dtype) else g.dtype
         self.gate_up = Linear(torch.cat([g.to(wdt), u.to(wdt)], dim=0).to(device))
-        self.down = Linear(tensors["down_proj.weight"].to(device))
+        self.down = Linear(tensors[self.names[2]].to(device))
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         return self.down.partial(self.gate_up.swiglu(x))

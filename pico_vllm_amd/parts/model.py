@@ -9,7 +9,7 @@ from ..config.registry import load_model_description
 from ..ops import kernels
 from ..ops.linear import Linear
 from ..weights.loader import load_checkpoint
-from . import attention, attention_bias, block, mlp, moe, norm, positions, rotary  # noqa: F401  (register the parts)
+from . import attention, attention_bias, attention_gated, block, gla, mlp, moe, norm, positions, rotary  # noqa: F401  (register the parts)
 from .base import Block, StepContext
 from .registry import build_part, part_class
 from .spec import CacheSpec, ModelSpec, ParamSpec

@@ -84,3 +84,97 @@ class RoutedExperts(FeedForward):
 
     def graph_variant(self, ctx: StepContext) -> tuple:
         return (("routed_experts", kernels.moe_grouped_rows(ctx.num_tokens, self.top)),)
+
+
+@register_part("feed_forward", "softmax_routed_experts")
+class SoftmaxRoutedExperts(FeedForward):
+    """Router: z = x Wr^T in float32 over ``num_experts + identity`` outputs, scores s = softmax(z) over all of them.
+    The ``top`` outputs with the largest s + correction are chosen (the correction, a stored vector, only steers the
+    choice); the weights are the chosen s over their sum (+ 1e-20), times ``scale``.
+
+    Expert e < num_experts on a token x: Wd_e (silu(Wg_e x) * (Wu_e x)), no biases; the last ``identity`` router outputs
+    stand for experts without tensors that return x itself.  A token's output is the weighted sum of its experts'
+    outputs.  With ``shared_size`` > 0 one more gated feed-forward of that inner size runs for every token and is added.
+
+    The experts' matrices are stacked at load (gate_up [E, 2 F, D], down [E, D, F]); everything a step decides is
+    decided on the device.  ``forward`` returns the routed sum, or [routed sum, shared expert's output] (deltas that the
+    arrangement adds to the residual stream one after the other)."""
+    graph_safe_prompts = True
+
+    def __init__(self, hidden_size: int, expert_size: int, num_experts: int, top: int, identity: int = 0, scale: float = 1.0,
+                 shared_size: int = 0, correction_name: Optional[str] = "correction", router_name: str = "router",
+                 expert_names: tuple = ("e{}.gate", "e{}.up", "e{}.down"),
+                 shared_names: tuple = ("shared.gate", "shared.up", "shared.down"), act_dtype: torch.dtype = torch.bfloat16):
+        if num_experts < 1 or identity < 0 or not 1 <= top <= min(num_experts + identity, kernels.MOE_MAX_TOP):
+            raise ValueError(f"{top} experts per token of {num_experts} + {identity} (at most {kernels.MOE_MAX_TOP})")
+        self.hidden_size, self.expert_size, self.num_experts, self.top = hidden_size, expert_size, num_experts, top
+        self.identity, self.scale, self.shared_size = int(identity), float(scale), int(shared_size)
+        self.correction_name, self.router_name = correction_name, router_name
+        self.expert_names, self.shared_names = tuple(expert_names), tuple(shared_names)
+        self.act_dtype = act_dtype
+        self.router: Optional[Linear] = None
+        self.correction: Optional[torch.Tensor] = None
+        self.gate_up: Optional[Linear] = None       # [E * 2 F, D]
+        self.down: Optional[Linear] = None          # [E * D, F]
+        self.shared = None
+        if self.shared_size:
+            from .mlp import SwiGLUMLP
+            self.shared = SwiGLUMLP(hidden_size, self.shared_size, act_dtype=act_dtype, names=self.shared_names)
+
+    @property
+    def outputs(self) -> int:
+        return self.num_experts + self.identity
+
+    def param_specs(self) -> List[ParamSpec]:
+        D, F = self.hidden_size, self.expert_size
+        g, u, d = self.expert_names
+        out = []
+        for e in range(self.num_experts):
+            out += [ParamSpec(g.format(e), (F, D)), ParamSpec(u.format(e), (F, D)), ParamSpec(d.format(e), (D, F))]
+        out.append(ParamSpec(self.router_name, (self.outputs, D)))
+        if self.correction_name:
+            out.append(ParamSpec(self.correction_name, (self.outputs,), role="bias"))
+        if self.shared is not None:
+            out += self.shared.param_specs()
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor], device, dtype) -> None:
+        g, u, d = self.expert_names
+        E = self.num_experts
+        self.router = Linear(tensors[self.router_name].float().to(device))      # routed in float32 in both engines
+        if self.correction_name:
+            self.correction = tensors[self.correction_name].to(device=device, dtype=torch.float32).contiguous()
+        ws = [tensors[n.format(e)] for e in range(E) for n in (g, u)]
+        wdt = torch.float32 if dtype == torch.float32 or any(w.dtype == torch.float32 for w in ws) else torch.bfloat16
+        self.gate_up = Linear(torch.cat([w.to(wdt) for w in ws], dim=0).to(device))
+        self.down = Linear(torch.cat([tensors[d.format(e)].to(wdt) for e in range(E)], dim=0).to(device))
+        if self.shared is not None:
+            self.shared.load({n: tensors[n] for n in self.shared_names}, device, dtype)
+
+    def weight_bytes(self) -> int:
+        # what a step of one token streams: the router, ``top`` experts and the shared expert
+        per = (self.gate_up.weight.numel() + self.down.weight.numel()) * self.gate_up.weight.element_size() // self.num_experts
+        return self.router.weight.numel() * 4 + self.top * per + (self.shared.weight_bytes() if self.shared is not None else 0)
+
+    def flops(self, tokens: int, pairs: int) -> float:
+        D, F = self.hidden_size, self.expert_size
+        return 2.0 * tokens * (self.outputs * D + self.top * 3 * F * D) + (self.shared.flops(tokens, pairs) if self.shared is not None else 0.0)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext):
+        E, F, D = self.num_experts, self.expert_size, self.hidden_size
+        experts, weights = kernels.moe_router_softmax(x, self.router.weight, self.correction, self.top, self.scale)
+        gate_up = self.gate_up.weight.view(E, 2 * F, D)
+        down = self.down.weight.view(E, D, F)
+        xe = x if x.dtype == gate_up.dtype else x.to(gate_up.dtype)
+        if kernels.moe_fast_ok(xe, gate_up, down):
+            out = kernels.moe_experts(xe, gate_up, down, experts, weights, 0.0, 0.0, mode=kernels.MOE_SWIGLU)
+        else:
+            out = kernels.moe_experts_plain(xe, gate_up, down, experts, weights, 0.0, 0.0, mode=kernels.MOE_SWIGLU)
+        if self.identity:
+            kernels.moe_identity(xe, experts, weights, out, E)
+        if self.shared is None:
+            return out
+        return [out, self.shared.forward(x, ctx)]
+
+    def graph_variant(self, ctx: StepContext) -> tuple:
+        return (("softmax_routed_experts", kernels.moe_grouped_rows(ctx.num_tokens, self.top)),)

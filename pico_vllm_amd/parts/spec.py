@@ -62,13 +62,15 @@ class CacheSpec:
     kind "paged_kv": what ``page_tensors`` lists, per page of tokens (the mixer names the tensors
     and their layout inside a page; the cache only allocates them, one allocation a tensor and
     layer, and hands them to the mixer by name); ``window`` > 0 means only the last ``window``
-    positions are ever read again, so older pages can be given back early.
+    positions are ever read again, so older pages can be given back early; except that the first ``keep_first``
+    positions of a request stay readable whatever the window (their pages are never given back early).
     kind "state": a fixed-size tensor of ``state_shape`` per request.
     kind "none": nothing.
     Layers with equal specs share a pool of page ids and a block table per request.
     """
     kind: str = "none"
     window: int = 0
+    keep_first: int = 0
     page_tensors: Tuple[PageTensor, ...] = ()
     state_shape: Tuple[int, ...] = ()
     state_dtype: str = "float32"
