@@ -179,6 +179,19 @@ def route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tens
     return chosen, ws / (ws.sum(-1, keepdim=True) + 1e-20) * scale
 
 
+def route_margin(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], top: int) -> torch.Tensor:
+    """[n]: how far the last chosen output lies in front of the first rejected one, as a fraction of the larger of
+    their two scores (a small value: rounding may choose the other)."""
+    s = torch.softmax(h @ router.T, -1)
+    choice = s if correction is None else s + correction
+    if top >= s.shape[1]:
+        return torch.full((s.shape[0],), float("inf"), dtype=s.dtype)
+    order = torch.argsort(choice, dim=-1, descending=True, stable=True)
+    a, b = order[:, top - 1:top], order[:, top:top + 1]
+    gap = torch.gather(choice, 1, a) - torch.gather(choice, 1, b)
+    return (gap / (torch.maximum(torch.gather(s, 1, a), torch.gather(s, 1, b)) + 1e-9))[:, 0]
+
+
 def routed_mlp(h: torch.Tensor, w: Dict[str, torch.Tensor], f: dict) -> torch.Tensor:
     """Experts e0 .. e(E-1) are gated feed-forwards; the router's outputs E .. E + identity - 1 stand for experts that
     hand their input on unchanged.  A shared expert, if there is one, runs for every token."""
@@ -213,9 +226,10 @@ def sub(tensors: Dict[str, torch.Tensor], prefix: str) -> Dict[str, torch.Tensor
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.float64, layers_out: Optional[List] = None):
+def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.float64, layers_out: Optional[List] = None,
+            margins_out: Optional[List] = None):
     """Logits [n, vocab] of a whole sequence from position 0.  ``layers_out``: a list that gets the residual stream
-    after every layer."""
+    after every layer; ``margins_out``: one that gets ``route_margin`` of every routed layer."""
     t = {k: v.to(dtype) if v.is_floating_point() else v for k, v in tensors.items()}
     ids = torch.as_tensor(list(tokens), dtype=torch.long)
     n = len(ids)
@@ -239,7 +253,10 @@ def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.
             a = gla_mixer(h1, w, m, eps)
         else:
             raise ValueError(layer["type"])
-        x = x + (a + feed_forward(h2, sub(t, p + "mlp."), layer.get("mlp")))
+        f = layer.get("mlp")
+        if margins_out is not None and f is not None and f["kind"] == "moe":
+            margins_out.append(route_margin(h2, t[p + "mlp.router"], t.get(p + "mlp.correction"), f["router"]["top"]))
+        x = x + (a + feed_forward(h2, sub(t, p + "mlp."), f))
         if layers_out is not None:
             layers_out.append(x.clone())
     return rms_norm(x, t["final.norm"], eps) @ t["head"].T
@@ -308,7 +325,7 @@ def random_model(config: dict, seed: int = 0, dtype=torch.bfloat16, rank: int = 
         elif last == "embed":
             t = torch.randn(shape, generator=g) / float((config.get("embedding") or {}).get("scale", 1.0))
         elif last == "router":
-            t = torch.randn(shape, generator=g) * 2.0 / math.sqrt(shape[-1])
+            t = torch.randn(shape, generator=g) * 6.0 / math.sqrt(shape[-1])       # peaked scores: few close calls
         elif last == "a2":
             t = torch.randn(shape, generator=g) * 2.0 / math.sqrt(shape[-1])
         elif last in ("q", "k"):

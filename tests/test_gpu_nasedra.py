@@ -1,0 +1,568 @@
+"""The Nasedra decoder in the engine against the plain implementation: each mechanism's kernel alone, then whole
+prompts, decoding through the cache and the state, portions, mixed batches in a small pool with few state slots, crafted
+keys at the edges of windows, pages and kept first positions, long decoding, and greedy generation through the entry
+point."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import plain_nasedra as P
+from gpu_util import DEV
+from nasedra_configs import CONFIGS, model_dir, tensors_of
+
+pytestmark = pytest.mark.gpu
+
+# rms of a position's error over its logits (mean taken off), in units of the logits' own rms there
+BOUND = {"float32": 3e-5, "bfloat16": 5e-2}
+# In bfloat16 a token whose last chosen and first rejected router output lie within CLOSE_CALL (a fraction of their
+# scores) may get the other one than in the plain run, which is no fault.  What it changes reaches every later
+# position (a recurrent layer forgets nothing at once): those positions are only held to TAINTED_BOUND.
+CLOSE_CALL, TAINTED_BOUND = 0.08, 1.5
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def row_errors(got, want):
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    w = want - want.mean(-1, keepdims=True)
+    return np.sqrt((d ** 2).mean(-1)) / np.sqrt((w ** 2).mean(-1))
+
+
+_plain = {}
+
+
+def plain_logits(name, tokens):
+    key = (name, tuple(tokens))
+    if key not in _plain:
+        margins = []
+        _plain[key] = P.forward(CONFIGS[name][0], tensors_of(name), tokens, margins_out=margins).numpy()
+        close = torch.stack(margins).min(0).values < CLOSE_CALL if margins else torch.zeros(len(tokens), dtype=torch.bool)
+        _plain[key + ("tainted",)] = (torch.cumsum(close.long(), 0) > 0).tolist()
+    return _plain[key]
+
+
+def tainted(name, tokens, position):
+    plain_logits(name, tokens)
+    return _plain[(name, tuple(tokens), "tainted")][position]
+
+
+def replay(name, dtype, steps, max_tokens, page_size=16, max_live=4):
+    """Run ``steps`` ([(entries, end)], entries [(id, tokens, want)]) through the engine's trace replayer; returns
+    {(id, position): logits row} and the replayer."""
+    from pico_vllm_amd.engine.replay import TraceReplayer
+    rp = TraceReplayer(model_dir(name), dtype, max_tokens, page_size, max_live)
+    fed, rows = {}, {}
+    for k, (entries, end) in enumerate(steps):
+        out = rp.run_step({"step": k, "entries": [{"id": r, "tokens": t, "want": list(w)} for r, t, w in entries], "end": list(end)})
+        at = 0
+        for r, t, w in entries:
+            for x in w:
+                rows[(r, fed.get(r, 0) + x)] = out[at]
+                at += 1
+            fed[r] = fed.get(r, 0) + len(t)
+        for r in end:
+            fed.pop(r, None)
+        rp.runner.manager.check()
+    return rows, rp
+
+
+def compare(name, dtype, rows, reqs):
+    errs, clean = [], 0
+    for (rid, pos), got in rows.items():
+        toks = reqs[rid.split("#")[0]]
+        e = float(row_errors(got[None], plain_logits(name, toks)[pos][None])[0])
+        errs.append(e)
+        if dtype == "bfloat16" and tainted(name, toks, pos):
+            assert e <= TAINTED_BOUND, f"{name} {dtype}: {rid} position {pos}: {e:.3g}"
+        else:
+            clean += 1
+            assert e <= BOUND[dtype], f"{name} {dtype}: {rid} position {pos}: {e:.3g} > {BOUND[dtype]}"
+    assert clean > 0
+    assert np.median(errs) <= BOUND[dtype] / 2, f"{name} {dtype}: median {np.median(errs):.3g}"
+
+
+def requests(name, lengths, seed=0):
+    rng = random.Random(seed)
+    V = CONFIGS[name][0]["vocab"]
+    return {f"r{i}": [rng.randrange(V) for _ in range(n)] for i, n in enumerate(lengths)}
+
+
+def cut(tokens, sizes, tail=0):
+    """Portions of ``sizes`` (cycled) and then the last ``tail`` tokens one by one."""
+    out, at, k = [], 0, 0
+    body = len(tokens) - tail
+    while at < body:
+        n = min(sizes[k % len(sizes)], body - at)
+        out.append(n)
+        at += n
+        k += 1
+    return out + [1] * tail
+
+
+def alone(reqs, portions_of):
+    steps = []
+    for rid, toks in reqs.items():
+        at = 0
+        parts = portions_of(toks)
+        for i, n in enumerate(parts):
+            steps.append(([(rid, toks[at:at + n], range(n))], [rid] if i == len(parts) - 1 else []))
+            at += n
+    return steps
+
+
+def roundup(n, m=64):
+    return -(-n // m) * m
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# rotation over neighbouring pairs, and the store
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nq,nkv,dk,dv,rotary_dim,scaling", [(3, 1, 24, 40, 16, (4.0, 64, 8.0, 1.0)), (4, 2, 64, 32, 64, None),
+                                                          (2, 2, 10, 6, 2, None), (2, 1, 32, 16, 0, None)])
+def test_rotation_of_pairs_and_the_store(dtype, nq, nkv, dk, dv, rotary_dim, scaling):
+    from pico_vllm_amd.ops import kernels as K
+    from pico_vllm_amd.parts.rotary import scaled_frequencies
+    dt = DT[dtype]
+    g = torch.Generator().manual_seed(3)
+    T, Pg, pages = 37, 8, 9
+    cols = nq * dk + nkv * dk + nkv * dv + 5
+    x = torch.randn(T, cols, generator=g).to(dt)
+    pos = torch.randint(0, 5000, (T,), generator=g).int()
+    slots = torch.randperm(Pg * pages, generator=g)[:T].int()
+    slots[5] = -1
+    kc = torch.full((pages, nkv, Pg, dk), 7.0, dtype=dt, device=DEV)
+    vc = torch.full((pages, nkv, dv, Pg), 7.0, dtype=dt, device=DEV)
+    table = None
+    rot = None
+    if rotary_dim:
+        rot = {"dims": rotary_dim, "base": 10000.0}
+        if scaling:
+            rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+        f, mag = scaled_frequencies(rotary_dim, 10000.0, scaling)
+        table = K.rope_table(pos.to(DEV), torch.tensor(f, dtype=torch.float64).float().to(DEV), mag)
+    xd = x.to(DEV).clone()
+    K.rope_pairs_store(xd, 0, nq * dk, nq * dk + nkv * dk, table, rotary_dim, slots.to(DEV), kc, vc, nq, nkv, dk, dv)
+    x64 = x.double()
+    q = x64[:, :nq * dk].view(T, nq, dk)
+    k = x64[:, nq * dk:nq * dk + nkv * dk].view(T, nkv, dk)
+    v = x64[:, nq * dk + nkv * dk:nq * dk + nkv * dk + nkv * dv].view(T, nkv, dv)
+    if rot:
+        q, k = P.rotate_pairs(q, pos, rot), P.rotate_pairs(k, pos, rot)
+    # positions up to 5,000 with float32 angles: an angle is off by up to 5000 * 2^-24
+    tol = dict(rtol=0, atol=3e-3 if dtype == "float32" else 5e-2)
+    got = xd.cpu().double()
+    assert torch.allclose(got[:, :nq * dk].view(T, nq, dk), q, **tol)
+    assert torch.equal(got[:, nq * dk:], x64[:, nq * dk:])                         # keys, values and the rest of the row stay
+    kcc, vcc = kc.cpu().double(), vc.cpu().double()
+    seen = torch.zeros(pages, Pg, dtype=torch.bool)
+    for t in range(T):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        seen[s // Pg, s % Pg] = True
+        assert torch.allclose(kcc[s // Pg, :, s % Pg, :], k[t], **tol)
+        assert torch.equal(vcc[s // Pg, :, :, s % Pg], v[t])
+        if rot and rotary_dim < dk:
+            assert torch.equal(kcc[s // Pg, :, s % Pg, rotary_dim:], k[t][:, rotary_dim:])
+    assert bool((kcc.permute(0, 2, 1, 3)[~seen] == 7.0).all()) and bool((vcc.permute(0, 3, 1, 2)[~seen] == 7.0).all())
+    # a layer that reads another layer's cache turns its queries only
+    xq = x.to(DEV).clone()
+    K.rope_pairs_store(xq, 0, 0, 0, table, rotary_dim, None, None, None, nq, nkv, dk, dv)
+    assert torch.equal(xq.cpu()[:, :nq * dk], xd.cpu()[:, :nq * dk]) and torch.equal(xq.cpu()[:, nq * dk:], x[:, nq * dk:])
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# attention: a cap on the scores, a window with kept first positions, a gate
+# ---------------------------------------------------------------------------------------------------------------
+def paged(k, v, P_, pages, dtype, seed=0, first_needed=0, keep=0):
+    """k [n, G, dk], v [n, G, dv] of one sequence into pages in random order, garbage elsewhere; pages that hold only
+    positions in [keep, first_needed) are marked as given back (-1) and hold garbage too."""
+    g = torch.Generator().manual_seed(seed)
+    n, G, dk = k.shape
+    dv = v.shape[2]
+    K = torch.randn(pages, G, P_, dk, generator=g) * 30
+    V = torch.randn(pages, G, dv, P_, generator=g) * 30
+    need = -(-n // P_)
+    perm = torch.randperm(pages, generator=g)[:need].tolist()
+    table = []
+    for j, page in enumerate(perm):
+        m = min(P_, n - j * P_)
+        if (j + 1) * P_ <= first_needed and j * P_ >= keep:
+            table.append(-1)
+            continue
+        table.append(page)
+        K[page, :, :m] = k[j * P_:j * P_ + m].transpose(0, 1)
+        V[page, :, :, :m] = v[j * P_:j * P_ + m].permute(1, 2, 0)
+    return K.to(DEV, dtype), V.to(DEV, dtype), torch.tensor([table], dtype=torch.int32, device=DEV)
+
+
+def plain_attention(q, k, v, positions, scale, cap, window, keep, gate):
+    """q [m, H, dk] at ``positions`` over keys k [n, G, dk], v [n, G, dv] at positions 0 .. n - 1."""
+    m, H, _ = q.shape
+    G = k.shape[1]
+    out = torch.zeros(m, H, v.shape[2], dtype=torch.float64)
+    for a, i in enumerate(positions):
+        js = [j for j in range(k.shape[0]) if P.visible(i, j, window, keep)]
+        for h in range(H):
+            g = h // (H // G)
+            s = P.capped(torch.stack([(q[a, h] * k[j, g]).sum() for j in js]) * scale, cap)
+            out[a, h] = torch.softmax(s, 0) @ v[js, g]
+    if gate is not None:
+        out = out * torch.sigmoid(gate.view_as(out))
+    return out
+
+
+ATTENTION_SHAPES = [  # H, G, dk, dv, page, window, keep, cap, gated
+    (4, 1, 64, 80, 16, 24, 6, 50.0, True), (8, 2, 64, 32, 8, 44, 5, None, True), (3, 1, 24, 40, 16, 12, 3, 30.0, True),
+    (4, 4, 32, 64, 16, None, 0, 15.0, False), (2, 1, 32, 16, 32, 5, 9, 5.0, True), (20, 1, 32, 16, 16, 70, 33, 10.0, True),
+    (6, 3, 10, 6, 8, 9, 1, None, True)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,dk,dv,Pg,window,keep,cap,gated", ATTENTION_SHAPES)
+def test_attention_kernels_over_prompts_portions_and_single_tokens(dtype, H, G, dk, dv, Pg, window, keep, cap, gated):
+    from pico_vllm_amd.ops import attention_bias_fast, kernels as K
+    dt = DT[dtype]
+    g = torch.Generator().manual_seed(H * 100 + dk)
+    n = 150
+    q = (torch.randn(n, H, dk, generator=g) * 1.5).to(dt)
+    k = (torch.randn(n, G, dk, generator=g) * 1.5).to(dt)
+    v = torch.randn(n, G, dv, generator=g).to(dt)
+    gate = torch.randn(n, H * dv, generator=g).to(dt) if gated else None
+    scale = 0.9 * dk ** -0.5
+    want = plain_attention(q.double(), k.double(), v.double(), range(n), scale, cap, window, keep,
+                           gate.double() if gated else None).view(n, H * dv)
+    kernels_ = ["plain"]
+    fast = None
+    if dtype == "bfloat16" and attention_bias_fast.supported(dk, dv):
+        fast = attention_bias_fast.FastBiasAttention(H, G, dk, dv, scale, window or 0, softcap=cap or 0.0, keep_first=keep, gated=gated)
+        kernels_ += ["fast", "fast_split", "fast_pieces"]
+    # one row holds q and, behind a gap, the gate (rows with a stride, as the mixer's product leaves them)
+    row = torch.zeros(n, H * dk + 8 + H * dv, dtype=dt)
+    row[:, :H * dk] = q.view(n, -1)
+    if gated:
+        row[:, H * dk + 8:] = gate
+    row = row.to(DEV)
+    for first, count in ((0, n), (0, 1), (0, 7), (61, 40), (n - 1, 1), (n - 2, 2), (37, 1), (100, 50)):
+        hi = first + count
+        first_needed = max(0, first - window + 1) if window else 0
+        Kc, Vc, bt = paged(k[:hi], v[:hi], Pg, 40, dt, seed=first, first_needed=first_needed, keep=keep if window else 0)
+        pos = torch.arange(first, hi, dtype=torch.int32, device=DEV)
+        seq = torch.zeros(count, dtype=torch.int32, device=DEV)
+        cu = torch.tensor([0, count], dtype=torch.int32, device=DEV)
+        rows = row[first:hi]
+        gt = rows[:, H * dk + 8:] if gated else None
+        for which in kernels_:
+            if which == "plain":
+                got = K.attn_bias_plain(rows, Kc, Vc, bt, pos, seq, H, G, dk, dv, scale, window or 0, softcap=cap or 0.0,
+                                        keep_first=keep, gate=gt)
+            else:
+                got = fast.run(rows, Kc, Vc, bt, cu, pos, 1, split={"fast": False, "fast_split": True, "fast_pieces": True}[which],
+                               chunks={"fast": 1, "fast_split": 1, "fast_pieces": 3}[which], gate=gt)
+            err = (got.double().cpu() - want[first:hi]).abs().max().item()
+            assert err <= (2e-5 if dtype == "float32" else 4e-2), (which, first, count, err)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("Pg", [8, 32])
+def test_one_key_that_stands_out_at_every_edge(dtype, Pg):
+    """All keys but one are nearly orthogonal to the query; the one carries a value of its own.  Placed just inside and
+    just outside the window, at the last kept first position and right behind it, at page borders and far back, the
+    output says whether the query saw it; as part of a prompt and as a single token."""
+    from pico_vllm_amd.ops import attention_bias_fast, kernels as K
+    dt = DT[dtype]
+    H, G, dk, dv, window, keep = 4, 2, 32, 16, 40, 5
+    n = 400
+    g = torch.Generator().manual_seed(5)
+    scale = 1.0
+    fast = attention_bias_fast.FastBiasAttention(H, G, dk, dv, scale, window, softcap=30.0, keep_first=keep) if dtype == "bfloat16" else None
+    i = n - 1
+    cases = [(i - window + 1, True), (i - window, False), (keep - 1, True), (keep, False), (0, True), (i - 8, True), (i - 16, True),
+             (i - 32, True), (i, True), (200, False), (Pg, False), (Pg - 1, False), (2 * Pg, False)]
+    for j, seen in cases:
+        k = torch.randn(n, G, dk, generator=g) * 0.05
+        v = torch.randn(n, G, dv, generator=g) * 0.1
+        q = torch.randn(n, H, dk, generator=g) * 0.05
+        q[i] = 0.0
+        q[i, :, 0] = 4.0
+        k[j, :, 0] = 4.0                       # score 16 against scores near 0
+        v[j] = 5.0
+        for first in (i, i - 70):              # a single token; the end of a portion of 71 tokens
+            count = i + 1 - first
+            Kc, Vc, bt = paged(k.to(dt), v.to(dt), Pg, 64, dt, seed=j, first_needed=max(0, first - window + 1), keep=keep)
+            pos = torch.arange(first, i + 1, dtype=torch.int32, device=DEV)
+            seq = torch.zeros(count, dtype=torch.int32, device=DEV)
+            rows = q[first:].reshape(count, H * dk).to(DEV, dt)
+            outs = [K.attn_bias_plain(rows, Kc, Vc, bt, pos, seq, H, G, dk, dv, scale, window, softcap=30.0, keep_first=keep)]
+            if fast is not None:
+                cu = torch.tensor([0, count], dtype=torch.int32, device=DEV)
+                outs += [fast.run(rows, Kc, Vc, bt, cu, pos, 1, split=s, chunks=c) for s, c in ((False, 1), (True, 1), (True, 2))]
+            for o in outs:
+                last = o[-1].float().cpu()
+                if seen:
+                    assert float(last.min()) > 4.5, (j, first, last)
+                else:
+                    assert float(last.abs().max()) < 0.5, (j, first, last)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# gated linear attention
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,dk,dv,rank,tau", [(2, 24, 40, 5, 4.0), (4, 64, 64, 16, 16.0), (1, 80, 100, 3, 1.0), (3, 16, 8, 2, 30.0),
+                                              (2, 256, 72, 8, 8.0)])
+def test_gla_kernels_in_portions_and_token_by_token(dtype, H, dk, dv, rank, tau):
+    from pico_vllm_amd.ops import kernels as K
+    dt = DT[dtype]
+    g = torch.Generator().manual_seed(dk)
+    lens = [53, 1, 20]
+    T = sum(lens)
+    cols = [H * dk, H * dk, H * dv, H * dv, rank]
+    offs = np.cumsum([0] + cols).tolist()
+    x = torch.randn(T, offs[-1], generator=g).to(dt)
+    a2 = (torch.randn(H * dk, rank, generator=g) * 1.5).to(dt)
+    b = 1.0 + 2.0 * torch.randn(H * dk, generator=g)
+    w = 1.0 + 0.2 * torch.randn(dv, generator=g)
+    eps = 1e-5
+    x64 = x.double()
+    z = x64[:, offs[4]:] @ a2.double().T + b.double()
+    alpha = torch.sigmoid(z).pow(1.0 / tau).view(T, H, dk)
+    q = x64[:, :offs[1]].view(T, H, dk) * dk ** -0.5
+    k = x64[:, offs[1]:offs[2]].view(T, H, dk)
+    v = x64[:, offs[2]:offs[3]].view(T, H, dv)
+    gate = x64[:, offs[3]:offs[4]]
+    want_o, want_S, at = [], [], 0
+    for n in lens:
+        o, S = P.gla_recurrence(q[at:at + n], k[at:at + n], v[at:at + n], alpha[at:at + n])
+        want_o.append(o)
+        want_S.append(S)
+        at += n
+    want_o = torch.cat(want_o)
+    want_out = (P.rms_norm(want_o, w.double(), eps).reshape(T, H * dv) * P.silu(gate))
+    xd = x.to(DEV)
+    ld = K.gla_decay(xd, offs[4], a2.to(DEV), b.to(DEV), tau)
+    assert torch.allclose(ld.cpu().double().exp(), alpha.view(T, -1), rtol=2e-5 if dtype == "float32" else 1e-4, atol=1e-7)
+    slots_of = [2, 0, 3]                       # of 4 slots and the spare one
+    tol = dict(rtol=2e-4, atol=2e-4) if dtype == "float32" else dict(rtol=2e-3, atol=2e-3)      # the inputs are the same bits
+    for parts in ([1.0], [0.5, 0.5], None):    # whole; two halves; token by token
+        state = torch.full((5, H, dk, dv), 3.0, device=DEV)
+        for s in slots_of:
+            state[s] = 0
+        outs = [torch.zeros(n, H * dv) for n in lens]
+        done = [0] * len(lens)
+        while any(d < n for d, n in zip(done, lens)):
+            step = []
+            for bi, n in enumerate(lens):
+                if done[bi] >= n:
+                    continue
+                m = 1 if parts is None else max(1, int(round(n * parts[0])))
+                m = min(m, n - done[bi])
+                step.append((bi, done[bi], m))
+            rows = torch.cat([torch.arange(sum(lens[:bi]) + d, sum(lens[:bi]) + d + m) for bi, d, m in step])
+            cu = torch.tensor(np.cumsum([0] + [m for _, _, m in step]), dtype=torch.int32, device=DEV)
+            sl = torch.tensor([slots_of[bi] for bi, _, _ in step], dtype=torch.int32, device=DEV)
+            xs = xd[rows.to(DEV)].contiguous()
+            o = K.gla_scan(xs, 0, offs[1], offs[2], ld[rows.to(DEV)].contiguous(), cu, sl, state, len(step), H, dk, dv, dk ** -0.5)
+            a = 0
+            for bi, d, m in step:
+                outs[bi][d:d + m] = o[a:a + m].cpu()
+                a += m
+                done[bi] += m
+        got = torch.cat(outs).double()
+        assert torch.allclose(got, want_o.view(T, -1), **tol), (parts, (got - want_o.view(T, -1)).abs().max())
+        for bi, s in enumerate(slots_of):
+            assert torch.allclose(state[s].cpu().double(), want_S[bi], **tol)
+        assert bool((state[1] == 3.0).all()) and bool((state[4] == 3.0).all())          # other slots are not touched
+        if parts == [1.0]:
+            whole = got
+        elif dtype == "float32":
+            assert torch.equal(got, whole)     # the same bits however the sequences were cut
+    out = K.gla_out(torch.cat(outs).to(DEV), xd, offs[3], w.to(DEV), eps, H, dv)
+    ref = (P.rms_norm(torch.cat(outs).double().view(T, H, dv), w.double(), eps).reshape(T, H * dv) * P.silu(gate))
+    assert torch.allclose(out.cpu().double(), ref, rtol=1e-5 if dtype == "float32" else 1e-2, atol=1e-5 if dtype == "float32" else 1e-2)
+    assert torch.allclose(ref, want_out, rtol=1e-2, atol=1e-2)
+
+
+def test_a_decay_near_one_keeps_a_far_token_in_the_state():
+    """With decays of almost 1 the value of the first token still dominates the output 600 tokens later; with fast
+    decays it is gone."""
+    from pico_vllm_amd.ops import kernels as K
+    H, dk, dv, T = 1, 32, 64, 600
+    for bias, kept in ((12.0, True), (-2.0, False)):
+        x = torch.zeros(T, 2 * dk + 2 * dv + 1)
+        x[:, 0] = dk ** 0.5                     # q: channel 0
+        x[0, dk] = 1.0                          # k of the first token: channel 0
+        x[0, 2 * dk:2 * dk + dv] = 7.0          # its value
+        a2 = torch.zeros(dk, 1)
+        ld = K.gla_decay(x.to(DEV), 2 * dk + 2 * dv, a2.to(DEV), torch.full((dk,), bias, device=DEV), 1.0)
+        state = torch.zeros(2, H, dk, dv, device=DEV)
+        o = K.gla_scan(x.to(DEV), 0, dk, 2 * dk, ld, torch.tensor([0, T], dtype=torch.int32, device=DEV),
+                       torch.tensor([0], dtype=torch.int32, device=DEV), state, 1, H, dk, dv, dk ** -0.5)
+        last = float(o[-1, 0])
+        want = 7.0 * torch.sigmoid(torch.tensor(bias, dtype=torch.float64)).item() ** (T - 1)
+        assert last == pytest.approx(want, rel=1e-3, abs=1e-6)
+        assert (last > 6.5) == kept
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# routing and experts
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("E,ident,top,scale,T,D", [(5, 2, 2, 1.5, 33, 72), (6, 1, 3, 1.0, 200, 128), (3, 0, 1, 1.0, 9, 96), (8, 3, 4, 2.0, 70, 40),
+                                                 (4, 2, 1, 0.7, 130, 128)])
+def test_softmax_router_choice_and_weights(E, ident, top, scale, T, D):
+    from pico_vllm_amd.ops import kernels as K
+    g = torch.Generator().manual_seed(E)
+    x = torch.randn(T, D, generator=g)
+    wr = torch.randn(E + ident, D, generator=g) * 3.0 / D ** 0.5
+    corr = 0.05 * torch.randn(E + ident, generator=g)
+    for c in (corr, None):
+        chosen, w = P.route(x.double(), wr.double(), None if c is None else c.double(), top, scale)
+        ge, gw = K.moe_router_softmax(x.to(DEV), wr.to(DEV), None if c is None else c.to(DEV), top, scale)
+        margin = P.route_margin(x.double(), wr.double(), None if c is None else c.double(), top)
+        sure = margin > 1e-4
+        assert bool(sure.float().mean() > 0.9)
+        assert torch.equal(ge.cpu().long()[sure], chosen[sure])
+        assert torch.allclose(gw.cpu().double()[sure], w[sure], rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("E,ident,top,F,D,T,shared", [(5, 2, 2, 32, 72, 19, 48), (6, 1, 3, 64, 128, 300, 0), (4, 2, 1, 32, 128, 90, 64),
+                                                     (3, 0, 1, 40, 96, 7, 0), (8, 3, 4, 24, 40, 50, 16)])
+def test_experts_with_pass_through_outputs_and_a_shared_expert(dtype, E, ident, top, F, D, T, shared):
+    """The part against the plain feed-forward, routing by the plain choice where the two could differ."""
+    from pico_vllm_amd.parts.base import StepContext
+    from pico_vllm_amd.parts.moe import SoftmaxRoutedExperts
+    dt = DT[dtype]
+    g = torch.Generator().manual_seed(F)
+    f = {"kind": "moe", "expert": {"ff": F}, "router": {"experts": E, "top": top, "identity": ident, "scale": 1.3}}
+    if shared:
+        f["shared"] = {"ff": shared}
+    w = {"router": (torch.randn(E + ident, D, generator=g) * 4.0 / D ** 0.5).to(torch.bfloat16),
+         "correction": (0.05 * torch.randn(E + ident, generator=g)).to(torch.bfloat16)}
+    for e in range(E):
+        w.update({f"e{e}.gate": (torch.randn(F, D, generator=g) / D ** 0.5).to(torch.bfloat16),
+                  f"e{e}.up": (torch.randn(F, D, generator=g) / D ** 0.5).to(torch.bfloat16),
+                  f"e{e}.down": (torch.randn(D, F, generator=g) / F ** 0.5).to(torch.bfloat16)})
+    if shared:
+        w.update({"shared.gate": (torch.randn(shared, D, generator=g) / D ** 0.5).to(torch.bfloat16),
+                  "shared.up": (torch.randn(shared, D, generator=g) / D ** 0.5).to(torch.bfloat16),
+                  "shared.down": (torch.randn(D, shared, generator=g) / shared ** 0.5).to(torch.bfloat16)})
+    part = SoftmaxRoutedExperts(D, F, E, top, identity=ident, scale=1.3, shared_size=shared, act_dtype=dt)
+    assert {p.name: tuple(p.shape) for p in part.param_specs()} == {k: tuple(v.shape) for k, v in w.items()}
+    part.load({k: (v.float() if dtype == "float32" else v) for k, v in w.items()}, torch.device(DEV), dt)
+    x = torch.randn(T, D, generator=g).to(dt)
+    want = P.routed_mlp(x.double(), {k: v.double() for k, v in w.items()}, f)
+    sure = P.route_margin(x.double(), w["router"].double(), w["correction"].double(), top) > (1e-4 if dtype == "float32" else 0.05)
+    out = part.forward(x.to(DEV), None)
+    total = torch.zeros(T, D, dtype=torch.float64)
+    for delta in (out if isinstance(out, (list, tuple)) else [out]):
+        d = delta.double().cpu()
+        total += d.sum(0) if d.dim() == 3 else d
+    assert bool(sure.float().mean() > 0.7)
+    err = (total - want)[sure].abs().max().item()
+    assert err <= (1e-4 if dtype == "float32" else 6e-2) * max(1.0, float(want.abs().max())), err
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# whole models through the replayer
+# ---------------------------------------------------------------------------------------------------------------
+PAGE = {"a": 16, "b": 8, "c": 32}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_whole_prompts_and_token_by_token_from_the_first_token(name, dtype):
+    reqs = requests(name, [150, 1, 37], seed=1)
+    rows, _ = replay(name, dtype, alone(reqs, lambda t: [len(t)]), roundup(150), PAGE[name])
+    compare(name, dtype, rows, reqs)
+    one = {"r2": reqs["r2"]}
+    rows1, _ = replay(name, dtype, alone(one, lambda t: [1] * len(t)), roundup(37), PAGE[name])
+    compare(name, dtype, rows1, one)
+    if dtype == "float32":
+        for key, row in rows1.items():
+            assert np.array_equal(row, rows[key])         # decoded through cache and state: the same bits as the prompt
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_portions_of_many_sizes_and_decoding_over_every_edge(name, dtype):
+    """Portions of 2 to 70 tokens, then 60 single tokens: windows of 12 to 100, kept first positions and pages of 8 to 32
+    tokens are all passed while decoding."""
+    reqs = requests(name, [190], seed=2)
+    rows, _ = replay(name, dtype, alone(reqs, lambda t: cut(t, [2, 33, 5, 70, 3, 16], tail=60)), roundup(190), PAGE[name])
+    compare(name, dtype, rows, reqs)
+    if dtype == "float32":
+        whole, _ = replay(name, dtype, alone(reqs, lambda t: [len(t)]), roundup(190), PAGE[name])
+        for key, row in rows.items():
+            assert np.array_equal(row, whole[key])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_mixed_batches_in_a_pool_that_holds_what_is_live(name, dtype):
+    """Seven unequal requests, at most three live: portions of some beside single tokens of others, in a pool that holds
+    just the live ones and with three state slots, so that pages and slots are used again; each request against itself alone."""
+    lengths = [70, 33, 120, 9, 64, 47, 101]
+    reqs = requests(name, lengths, seed=4)
+    rng = random.Random(7)
+    waiting, live, done_at, steps = list(reqs), {}, {}, []
+    sizes = [17, 2, 40, 6, 29]
+    peak = 0
+    while waiting or live:
+        while waiting and len(live) < 3:
+            live[waiting.pop(0)] = 0
+        entries, end = [], []
+        for rid in list(live):
+            toks, at = reqs[rid], live[rid]
+            if rng.random() < 0.2 and len(live) > 1:
+                continue                                        # left out of this step
+            tail = len(toks) - at <= 12
+            n = 1 if tail else min(sizes[rng.randrange(len(sizes))], len(toks) - 12 - at)
+            entries.append((rid, toks[at:at + n], range(n)))
+            live[rid] = at + n
+            if live[rid] == len(toks):
+                end.append(rid)
+        peak = max(peak, sum(roundup(live[r], PAGE[name]) for r in live))
+        for rid in end:
+            del live[rid]
+        if entries:
+            steps.append((entries, end))
+    rows, rp = replay(name, dtype, steps, roundup(peak), PAGE[name], max_live=3)
+    compare(name, dtype, rows, reqs)
+    assert rp.runner.manager.num_free_pages() == rp.runner.manager.groups[0].pool.num_pages       # all given back
+    if dtype == "float32":
+        solo, _ = replay(name, dtype, alone(reqs, lambda t: [len(t)]), roundup(max(lengths)), PAGE[name])
+        for key, row in rows.items():
+            assert np.array_equal(row, solo[key])               # what else is in the batch changes no bit
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(dtype):
+    reqs = requests("b", [330], seed=6)
+    steps = alone(reqs, lambda t: cut(t, [30], tail=300))
+    rows, _ = replay("b", dtype, steps, roundup(330), PAGE["b"])
+    compare("b", dtype, rows, reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("graphs", [False, True])
+def test_greedy_generation_through_the_entry_point(dtype, graphs):
+    from pico_vllm_amd import LLM, SamplingParams
+    name = "b"
+    prompts = [[5, 17, 3, 200, 41], [9] * 19, [77, 2], list(range(60, 130)), [1], [250, 3, 3, 8, 100, 100]]
+    llm = LLM(model=model_dir(name), dtype=dtype, block_size=8, num_gpu_blocks=48, max_seq_len=160, max_num_seqs=3,
+              max_num_batched_tokens=24, use_cuda_graph=graphs, max_batch_size=4)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=12, temperature=0.0, ignore_eos=True))
+    cfg, t = CONFIGS[name][0], tensors_of(name)
+    for p, o in zip(prompts, outs):
+        assert len(o.token_ids) == 12
+        toks = list(p)
+        for tok in o.token_ids:
+            logits = P.forward(cfg, t, toks)[-1]
+            slack = 1e-4 if dtype == "float32" else 0.08 * float(logits.std())
+            assert float(logits[tok]) >= float(logits.max()) - slack, (dtype, p, o.token_ids, tok, int(logits.argmax()))
+            toks.append(tok)
+    llm.engine.runner.manager.check()
