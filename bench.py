@@ -7,8 +7,9 @@
                                                             (64 requests, prompts of 128..4096 tokens, 256 new tokens each,
                                                              continuous batching with prompts cut into portions)
 
-  python bench.py --workload designs --layers 4             (Lerazen beside the Qwen2.5 shape of equal size, at two sizes:
-                                                             decode at batch 1 and 8, the 2,048-token prefill)
+  python bench.py --workload designs --layers 4             (Lerazen and Nasedra, each beside the Qwen2.5 shape of equal size,
+                                                             at two sizes: decode at batch 1 and 8, the 2,048-token
+                                                             prefill; --designs nasedra measures that design's pairs only)
 
   python bench.py --workload long --shape 32b --device-weights --context 32768
                                                             (one 16k-token prompt in portions of 2,048, then decode at
@@ -52,9 +53,11 @@ from pico_vllm_amd.config.presets import preset   # noqa: E402  (needs ROOT on t
 SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", preset("1.5b")), "7b": ("Qwen2.5-7B shape", preset("7b")),
           "32b": ("Qwen2.5-32B shape", preset("32b")),
           "lerazen-1.5b": ("Lerazen at the 1.5B shape's sizes", preset("lerazen-1.5b")),
-          "lerazen-7b": ("Lerazen at the 7B shape's sizes", preset("lerazen-7b"))}
+          "lerazen-7b": ("Lerazen at the 7B shape's sizes", preset("lerazen-7b")),
+          "nasedra-1.5b": ("Nasedra at the 1.5B shape's sizes", preset("nasedra-1.5b")),
+          "nasedra-7b": ("Nasedra at the 7B shape's sizes", preset("nasedra-7b"))}
 # --workload designs: (a design's configuration, the closest existing model at equal size)
-DESIGN_PAIRS = (("lerazen-1.5b", "1.5b"), ("lerazen-7b", "7b"))
+DESIGN_PAIRS = (("lerazen-1.5b", "1.5b"), ("lerazen-7b", "7b"), ("nasedra-1.5b", "1.5b"), ("nasedra-7b", "7b"))
 CONFIG = SHAPES["1.5b"][1]   # the shape being measured (set in main)
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
@@ -413,9 +416,9 @@ def design_points(dtype, layers, steps, warmup, only=None):
     import torch
     rows = []
     for pair in DESIGN_PAIRS:
+        if only and not any(pair[0].startswith(o) for o in only):
+            continue
         for key in pair:
-            if only and key not in only:
-                continue
             name, raw = SHAPES[key]
             arch, typed, _ = describe(raw)
             cut = arch.with_layers(raw, layers) if layers else raw
@@ -457,6 +460,7 @@ def main() -> int:
                     "architecture) instead of writing random weights of --shape")
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (default: the 1.5B shape)")
     ap.add_argument("--layers", type=int, default=0, help="run only this many layers of the shape (0: all)")
+    ap.add_argument("--designs", default="", help="with --workload designs: only the pairs of these designs (names' beginnings, commas between them)")
     ap.add_argument("--context", type=int, default=4096, help="context length at which the decode steps end")
     ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "sweep", "designs"],
                     help="decode: the contract's steady decode steps; serve: many requests of mixed lengths at once; "
@@ -530,7 +534,8 @@ def main() -> int:
                           "p": top_p}))
         return 0
     if a.workload == "designs":
-        rows = design_points(a.dtype, a.layers, min(a.steps, 100), min(a.warmup, 10))
+        rows = design_points(a.dtype, a.layers, min(a.steps, 100), min(a.warmup, 10),
+                             only=[x for x in a.designs.split(",") if x] or None)
         print(json.dumps({"metric": f"designs side by side: decode tok/s at batch 1 and 8 (context {CONTEXT}), prefill of {PREFILL_TOKENS} tokens",
                           "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
                           "data": "synthetic: random weights N(0, 0.02) drawn on the GPU, uniform random token ids",

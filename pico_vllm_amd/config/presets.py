@@ -49,6 +49,36 @@ DESIGN_PRESETS: Dict[str, Dict] = {
 }
 
 
+def _nasedra(vocab, width, layers, heads, kv_heads, dim, dense_ff, experts, top, expert_ff, shared_ff, gla_dim=64,
+             window=1024, keep_first=4) -> Dict:
+    """A Nasedra configuration of a real model's proportions, in groups of four layers: windowed attention with a dense
+    feed-forward, a recurrent layer with a routed one, attention over the first layer's keys and values with a dense
+    one, a recurrent layer with a routed one."""
+    rot = {"dims": dim, "base": 500000.0, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+
+    def attention(i):
+        m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 50.0,
+             "mask": {"size": window, "keep_first": keep_first}, "rot": rot}
+        if i % 4 == 2:
+            m["kv_from"] = i - 2
+        return m
+    recurrent = {"heads": heads, "dim": gla_dim, "vdim": dim, "tau": 16.0}
+    dense = {"kind": "dense", "ff": dense_ff}
+    routed = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "identity": 2, "scale": 1.5},
+              "shared": {"ff": shared_ff}}
+    return {"architecture": "Nasedra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": width ** 0.5},
+            "layers": [{"type": "gla", "mixer": recurrent, "mlp": routed} if i % 2 else
+                       {"type": "attention", "mixer": attention(i), "mlp": dense} for i in range(layers)]}
+
+
+# Nasedra at the sizes of the Qwen2.5 shapes: the same width, heads and layers, the same dense feed-forward; where it
+# is routed a token multiplies as many feed-forward weights (``top`` experts and the shared one).
+DESIGN_PRESETS.update({
+    "nasedra-1.5b": _nasedra(151936, 1536, 28, 12, 2, 128, 8960, 16, 2, 2240, 4480),
+    "nasedra-7b": _nasedra(152064, 3584, 28, 28, 4, 128, 18944, 32, 4, 2368, 9472),
+})
+
+
 def preset(name: str) -> Dict:
     import copy
     key = name.lower()

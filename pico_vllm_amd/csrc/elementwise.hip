@@ -187,6 +187,87 @@ extern "C" int pico_add_rmsnorm(float* resid, const void* delta, int delta_dtype
   return 0;
 }
 
+// Two norms of one row in one launch: resid[t] += delta[t] (if delta; `slabs` partial sums as above), then
+// out1[t] = norm(resid[t]) * w1 and out2[t] = norm(resid[t]) * w2, for an arrangement whose two sublayers read the same
+// stream through norms of their own.  One workgroup per row; the row is read again for the scaling (from the caches).
+template <typename TD, typename TO, bool VEC>
+__global__ void add_rmsnorm2_kernel(float* __restrict__ resid, const TD* __restrict__ delta, const float* __restrict__ w1,
+                                    const float* __restrict__ w2, TO* __restrict__ out1, TO* __restrict__ out2, int H,
+                                    float eps, int slabs, size_t slab_stride) {
+  __shared__ float scratch[16];
+  float* x = resid + (size_t)blockIdx.x * H;
+  const TD* dl = delta ? delta + (size_t)blockIdx.x * H : nullptr;
+  TO* o1 = out1 + (size_t)blockIdx.x * H;
+  TO* o2 = out2 + (size_t)blockIdx.x * H;
+  float ss = 0.f;
+  if (VEC) {
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      float4 v = *reinterpret_cast<const float4*>(x + i);
+      if (dl) {
+        for (int s = 0; s < slabs; s++) {
+          const float4 d = load4_f32(dl + s * slab_stride + i);
+          v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        }
+        *reinterpret_cast<float4*>(x + i) = v;
+      }
+      ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = block_sum(ss, scratch);
+    const float r = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      const float4 v = *reinterpret_cast<const float4*>(x + i);
+      const float4 g = *reinterpret_cast<const float4*>(w1 + i), k = *reinterpret_cast<const float4*>(w2 + i);
+      store4_f32(o1 + i, make_float4(v.x * r * g.x, v.y * r * g.y, v.z * r * g.z, v.w * r * g.w));
+      store4_f32(o2 + i, make_float4(v.x * r * k.x, v.y * r * k.y, v.z * r * k.z, v.w * r * k.w));
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = x[i];
+    if (dl) {
+      for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
+      x[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float v = x[i] * r;
+    store_f32(o1 + i, v * w1[i]);
+    store_f32(o2 + i, v * w2[i]);
+  }
+}
+
+extern "C" int pico_add_rmsnorm2(float* resid, const void* delta, int delta_dtype, int slabs, long long slab_stride,
+                                 const float* w1, const float* w2, void* out1, void* out2, int out_dtype, int T, int H,
+                                 float eps, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && H > 0, "pico_add_rmsnorm2: bad sizes T=%d H=%d", T, H);
+  PICO_REQUIRE(slabs >= 1 && slabs <= MAX_SLABS && slab_stride >= 0, "pico_add_rmsnorm2: 1 to %d slabs, got %d", MAX_SLABS, slabs);
+  PICO_REQUIRE(eps > 0.f, "pico_add_rmsnorm2: eps must be positive");
+  if (T == 0) return 0;
+  const bool vec = H % 4 == 0 && ((uintptr_t)resid | (uintptr_t)w1 | (uintptr_t)w2 | (uintptr_t)out1 | (uintptr_t)out2 |
+                                  (uintptr_t)delta) % 16 == 0 && slab_stride % 4 == 0;
+  const int threads = vec ? min(1024, max(64, (H / 4 + 63) / 64 * 64)) : (H >= 4096 ? 512 : (H >= 1024 ? 256 : 128));
+#define LAUNCH(TD, TO)                                                                                                   \
+  do {                                                                                                                   \
+    if (vec)                                                                                                             \
+      add_rmsnorm2_kernel<TD, TO, true><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w1, w2, (TO*)out1, (TO*)out2, \
+                                                                   H, eps, slabs, (size_t)slab_stride);                  \
+    else                                                                                                                 \
+      add_rmsnorm2_kernel<TD, TO, false><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w1, w2, (TO*)out1,          \
+                                                                    (TO*)out2, H, eps, slabs, (size_t)slab_stride);      \
+  } while (0)
+  if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_F32) LAUNCH(float, float);
+  else if (delta_dtype == PICO_DTYPE_BF16 && out_dtype == PICO_DTYPE_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_BF16) LAUNCH(float, bf16_t);
+  else if (delta_dtype == PICO_DTYPE_BF16 && out_dtype == PICO_DTYPE_F32) LAUNCH(bf16_t, float);
+  else PICO_REQUIRE(false, "pico_add_rmsnorm2: unknown dtypes %d %d", delta_dtype, out_dtype);
+#undef LAUNCH
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
 // resid[t] += delta[t] without a norm (for an arrangement that ends on an add)
 template <typename TD>
 __global__ void residual_add_kernel(float* __restrict__ resid, const TD* __restrict__ delta, size_t n) {

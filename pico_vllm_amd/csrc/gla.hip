@@ -55,17 +55,28 @@ extern "C" int pico_gla_decay(const void* x, int ldx, int dtype, const void* a2,
 // a thread keeps GLA_CPT state elements in registers over all tokens of the step.  Tokens are taken GLA_TB at a time:
 // their q, k and decays are staged in LDS (every thread reads all of its channels' from there), the waves' partial
 // outputs meet in LDS and are summed in wave order.
+//
+// Long portions are cut into chunks of `chunk` tokens that run side by side (the recurrence is linear in the state):
+//   GLA_LOCAL:  every chunk from a state of zero, no outputs; leaves its state in ws[chunk] and the sum of its decays'
+//               logarithms in ws_decay[chunk]
+//   (gla_combine_kernel walks a sequence's chunks: ws[j] <- the state in front of chunk j, and the slot's final state)
+//   GLA_FROM:   every chunk again from ws[chunk], writing the outputs
+// GLA_WHOLE is the plain walk from the slot's state (a sequence is one chunk).  blockIdx.x = sequence * max_chunks + chunk.
 // ---------------------------------------------------------------------------
 #define GLA_CPT 32
 #define GLA_TB 8
+#define GLA_WHOLE 0
+#define GLA_LOCAL 1
+#define GLA_FROM 2
 
-template <typename T>
+template <typename T, int MODE>
 __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, int ldx, int q_col, int k_col, int v_col,
                                                        const float* __restrict__ log_decay,
                                                        const int* __restrict__ cu_seqlens,
                                                        const int* __restrict__ state_slots, float* __restrict__ state,
                                                        float* __restrict__ out, int H, int dk, int dv, float qscale,
-                                                       int num_slots) {
+                                                       int num_slots, int chunk, int max_chunks, float* __restrict__ ws,
+                                                       float* __restrict__ ws_decay) {
   extern __shared__ float lds[];
   const int nw = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int CP = nw * GLA_CPT;                          // key channels with padding
@@ -73,16 +84,29 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
   float* ks = qs + GLA_TB * CP;
   float* as = ks + GLA_TB * CP;
   float* po = as + GLA_TB * CP;                         // [GLA_TB][nw][64]
-  const int b = blockIdx.x, h = blockIdx.y, v = blockIdx.z * 64 + lane;
+  const int b = MODE == GLA_WHOLE ? blockIdx.x : blockIdx.x / max_chunks, h = blockIdx.y, v = blockIdx.z * 64 + lane;
   const bool v_ok = v < dv;
-  const int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1];
+  int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1];
+  if (MODE != GLA_WHOLE) {
+    t_begin += (blockIdx.x % max_chunks) * chunk;
+    t_end = min(t_end, t_begin + chunk);
+  }
   const int slot = state_slots[b];
   if (slot < 0 || slot >= num_slots || t_end <= t_begin) return;
   const int c0 = wave * GLA_CPT;
-  float* sp = state + (((size_t)slot * H + h) * dk + c0) * dv + v;
+  float* sp = MODE == GLA_WHOLE ? state + (((size_t)slot * H + h) * dk + c0) * dv + v
+                                : ws + (((size_t)blockIdx.x * H + h) * dk + c0) * dv + v;
   float S[GLA_CPT];
 #pragma unroll
-  for (int c = 0; c < GLA_CPT; c++) S[c] = (v_ok && c0 + c < dk) ? sp[(size_t)c * dv] : 0.f;
+  for (int c = 0; c < GLA_CPT; c++) S[c] = (MODE != GLA_LOCAL && v_ok && c0 + c < dk) ? sp[(size_t)c * dv] : 0.f;
+  if (MODE == GLA_LOCAL && blockIdx.z == 0) {
+    // the chunk's decays multiplied up, as the sum of their logarithms, for the walk over the chunks
+    for (int c = threadIdx.x; c < dk; c += blockDim.x) {
+      float sum = 0.f;
+      for (int t = t_begin; t < t_end; t++) sum += log_decay[(size_t)t * H * dk + (size_t)h * dk + c];
+      ws_decay[((size_t)blockIdx.x * H + h) * dk + c] = sum;
+    }
+  }
 
   for (int t0 = t_begin; t0 < t_end; t0 += GLA_TB) {
     const int nb = min(GLA_TB, t_end - t0);
@@ -92,7 +116,7 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
       float qv = 0.f, kv = 0.f, av = 1.f;
       if (c < dk) {
         const T* row = x + (size_t)(t0 + tt) * ldx + (size_t)h * dk + c;
-        qv = load_f32(row + q_col) * qscale;
+        if (MODE != GLA_LOCAL) qv = load_f32(row + q_col) * qscale;
         kv = load_f32(row + k_col);
         av = expf(log_decay[(size_t)(t0 + tt) * H * dk + (size_t)h * dk + c]);
       }
@@ -112,14 +136,22 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
       float acc = 0.f;
 #pragma unroll
       for (int c = 0; c < GLA_CPT / 4; c++) {
-        const float4 av = a4[c], kv = k4[c], qv = q4[c];
-        S[4 * c + 0] = fmaf(av.x, S[4 * c + 0], kv.x * vv[tt]); acc = fmaf(S[4 * c + 0], qv.x, acc);
-        S[4 * c + 1] = fmaf(av.y, S[4 * c + 1], kv.y * vv[tt]); acc = fmaf(S[4 * c + 1], qv.y, acc);
-        S[4 * c + 2] = fmaf(av.z, S[4 * c + 2], kv.z * vv[tt]); acc = fmaf(S[4 * c + 2], qv.z, acc);
-        S[4 * c + 3] = fmaf(av.w, S[4 * c + 3], kv.w * vv[tt]); acc = fmaf(S[4 * c + 3], qv.w, acc);
+        const float4 av = a4[c], kv = k4[c];
+        S[4 * c + 0] = fmaf(av.x, S[4 * c + 0], kv.x * vv[tt]);
+        S[4 * c + 1] = fmaf(av.y, S[4 * c + 1], kv.y * vv[tt]);
+        S[4 * c + 2] = fmaf(av.z, S[4 * c + 2], kv.z * vv[tt]);
+        S[4 * c + 3] = fmaf(av.w, S[4 * c + 3], kv.w * vv[tt]);
+        if (MODE != GLA_LOCAL) {
+          const float4 qv = q4[c];
+          acc = fmaf(S[4 * c + 0], qv.x, acc);
+          acc = fmaf(S[4 * c + 1], qv.y, acc);
+          acc = fmaf(S[4 * c + 2], qv.z, acc);
+          acc = fmaf(S[4 * c + 3], qv.w, acc);
+        }
       }
-      po[(tt * nw + wave) * 64 + lane] = acc;
+      if (MODE != GLA_LOCAL) po[(tt * nw + wave) * 64 + lane] = acc;
     }
+    if (MODE == GLA_LOCAL) continue;
     __syncthreads();
     for (int i = threadIdx.x; i < nb * 64; i += blockDim.x) {
       const int tt = i >> 6, l = i & 63, vo = blockIdx.z * 64 + l;
@@ -129,34 +161,80 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
       out[(size_t)(t0 + tt) * H * dv + (size_t)h * dv + vo] = sum;
     }
   }
-  if (v_ok) {
+  if (MODE != GLA_FROM && v_ok) {
 #pragma unroll
     for (int c = 0; c < GLA_CPT; c++)
       if (c0 + c < dk) sp[(size_t)c * dv] = S[c];
   }
 }
 
+// The walk over a sequence's chunks, one thread per state element: ws[j] becomes the state in front of chunk j, the
+// slot gets the state behind the last chunk.  grid (sequences, heads, ceil(dk dv / 256)).
+__global__ __launch_bounds__(256) void gla_combine_kernel(const int* __restrict__ cu_seqlens,
+                                                          const int* __restrict__ state_slots, float* __restrict__ state,
+                                                          float* __restrict__ ws, const float* __restrict__ ws_decay, int H,
+                                                          int dk, int dv, int num_slots, int chunk, int max_chunks) {
+  const int b = blockIdx.x, h = blockIdx.y, e = blockIdx.z * 256 + threadIdx.x;
+  if (e >= dk * dv) return;
+  const int slot = state_slots[b], n = cu_seqlens[b + 1] - cu_seqlens[b];
+  if (slot < 0 || slot >= num_slots || n <= 0) return;
+  const int c = e / dv;
+  float* sp = state + ((size_t)slot * H + h) * dk * dv + e;
+  float S = *sp;
+  const int chunks = (n + chunk - 1) / chunk;
+  for (int j = 0; j < chunks; j++) {
+    const size_t at = (size_t)b * max_chunks + j;
+    float* w = ws + (at * H + h) * dk * dv + e;
+    const float local = *w;
+    *w = S;
+    S = fmaf(expf(ws_decay[(at * H + h) * dk + c]), S, local);
+  }
+  *sp = S;
+}
+
+// chunk == 0: every sequence walked whole from its slot.  chunk > 0: sequences cut into chunks of that many tokens that
+// run side by side (three launches); ws float32 [num_seqs * max_chunks, H, dk, dv], ws_decay [num_seqs * max_chunks, H, dk],
+// max_chunks at least the chunks of the longest sequence.
 extern "C" int pico_gla_scan(const void* x, int ldx, int dtype, int q_col, int k_col, int v_col, const float* log_decay,
                              const int* cu_seqlens, const int* state_slots, float* state, float* out, int num_seqs,
-                             int T, int H, int dk, int dv, float qscale, int num_slots, hipStream_t stream) {
+                             int T, int H, int dk, int dv, float qscale, int num_slots, int chunk, int max_chunks,
+                             float* ws, float* ws_decay, hipStream_t stream) {
   PICO_REQUIRE(num_seqs >= 0 && T >= 0 && H > 0 && dk > 0 && dv > 0 && num_slots > 0, "pico_gla_scan: bad sizes");
   PICO_REQUIRE(dk <= 8 * GLA_CPT, "pico_gla_scan: at most %d key channels a head, got %d", 8 * GLA_CPT, dk);
   PICO_REQUIRE(q_col >= 0 && k_col >= 0 && v_col >= 0 && ldx >= q_col + H * dk && ldx >= k_col + H * dk && ldx >= v_col + H * dv,
                "pico_gla_scan: the row of %d columns does not hold q, k and v", ldx);
-  PICO_REQUIRE(H <= 65535 && (dv + 63) / 64 <= 65535, "pico_gla_scan: sizes beyond the grid");
+  PICO_REQUIRE(H <= 65535 && (dv + 63) / 64 <= 65535 && (dk * dv + 255) / 256 <= 65535, "pico_gla_scan: sizes beyond the grid");
+  PICO_REQUIRE(chunk == 0 || (chunk > 0 && max_chunks > 0 && ws != nullptr && ws_decay != nullptr &&
+                              (long long)max_chunks * chunk >= T && (long long)num_seqs * max_chunks < (1ll << 31)),
+               "pico_gla_scan: chunks need room for their states and must cover the step's tokens");
   if (num_seqs == 0 || T == 0) return 0;
   const int nw = (dk + GLA_CPT - 1) / GLA_CPT;
   const size_t lds = (size_t)(3 * GLA_TB * nw * GLA_CPT + GLA_TB * nw * 64) * sizeof(float);
   PICO_REQUIRE(lds <= 64 * 1024, "pico_gla_scan: key channels beyond the staging memory");
-  const dim3 grid(num_seqs, H, (dv + 63) / 64);
-  if (dtype == PICO_DTYPE_F32)
-    gla_scan_kernel<float><<<grid, 64 * nw, lds, stream>>>((const float*)x, ldx, q_col, k_col, v_col, log_decay, cu_seqlens,
-                                                          state_slots, state, out, H, dk, dv, qscale, num_slots);
-  else if (dtype == PICO_DTYPE_BF16)
-    gla_scan_kernel<bf16_t><<<grid, 64 * nw, lds, stream>>>((const bf16_t*)x, ldx, q_col, k_col, v_col, log_decay, cu_seqlens,
-                                                           state_slots, state, out, H, dk, dv, qscale, num_slots);
-  else
+  const int vb = (dv + 63) / 64;
+#define GLA_LAUNCH(TT, MODE, GX)                                                                                          \
+  gla_scan_kernel<TT, MODE><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>((const TT*)x, ldx, q_col, k_col, v_col, log_decay,    \
+                                                                      cu_seqlens, state_slots, state, out, H, dk, dv, qscale, \
+                                                                      num_slots, chunk, max_chunks, ws, ws_decay)
+#define GLA_RUN(TT)                                                                                                        \
+  if (chunk == 0) {                                                                                                        \
+    GLA_LAUNCH(TT, GLA_WHOLE, num_seqs);                                                                                   \
+  } else {                                                                                                                 \
+    GLA_LAUNCH(TT, GLA_LOCAL, num_seqs * max_chunks);                                                                      \
+    gla_combine_kernel<<<dim3(num_seqs, H, (dk * dv + 255) / 256), 256, 0, stream>>>(cu_seqlens, state_slots, state, ws,   \
+                                                                                     ws_decay, H, dk, dv, num_slots, chunk, \
+                                                                                     max_chunks);                          \
+    GLA_LAUNCH(TT, GLA_FROM, num_seqs * max_chunks);                                                                       \
+  }
+  if (dtype == PICO_DTYPE_F32) {
+    GLA_RUN(float)
+  } else if (dtype == PICO_DTYPE_BF16) {
+    GLA_RUN(bf16_t)
+  } else {
     PICO_REQUIRE(false, "pico_gla_scan: unknown dtype %d", dtype);
+  }
+#undef GLA_RUN
+#undef GLA_LAUNCH
   PICO_LAUNCH_CHECK();
   return 0;
 }

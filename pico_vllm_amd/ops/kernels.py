@@ -140,6 +140,37 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     return out
 
 
+MAX_SLABS = 8           # partial sums that one norm launch adds up
+
+
+def add_rmsnorm2(resid: torch.Tensor, delta: Optional[torch.Tensor], weight1: torch.Tensor, weight2: torch.Tensor, eps: float,
+                 out_dtype: torch.dtype):
+    """resid += delta (if given; [T, H] or a float32 stack [S, T, H]), then the row's RMS norm with each of the two
+    weights: (norm(resid) * weight1, norm(resid) * weight2), one launch."""
+    _gpu(resid, delta, weight1, weight2)
+    T, H = resid.shape
+    if resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise KernelError("the residual stream must be contiguous float32")
+    for w in (weight1, weight2):
+        if w.dtype != torch.float32 or w.shape != (H,) or not w.is_contiguous():
+            raise KernelError(f"norm weight must be float32 of shape [{H}]")
+    slabs = 1
+    if delta is not None:
+        if delta.dim() == 3:
+            slabs = delta.shape[0]
+            if delta.dtype != torch.float32:
+                raise KernelError("a stack of partial sums must be float32")
+        if tuple(delta.shape[-2:]) != (T, H) or not delta.is_contiguous():
+            raise KernelError("delta must be contiguous and shaped like the residual stream")
+    out1 = torch.empty(T, H, dtype=out_dtype, device=resid.device)
+    out2 = torch.empty(T, H, dtype=out_dtype, device=resid.device)
+    lib = library.core()
+    _check(lib, lib.pico_add_rmsnorm2(_ptr(resid), _ptr(delta), _dt(delta) if delta is not None else F32, slabs, c_ll(T * H),
+                                      _ptr(weight1), _ptr(weight2), _ptr(out1), _ptr(out2), _DT[out_dtype], T, H, c_float(eps),
+                                      _stream()))
+    return out1, out2
+
+
 def residual_add(resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     _gpu(resid, delta)
     if resid.dtype != torch.float32 or not resid.is_contiguous() or delta.shape != resid.shape \
@@ -684,9 +715,11 @@ GLA_MAX_KEY_DIM = 256
 
 def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: torch.Tensor, cu_seqlens: torch.Tensor,
              state_slots: torch.Tensor, state: torch.Tensor, num_seqs: int, heads: int, dk: int, dv: int,
-             qscale: float) -> torch.Tensor:
+             qscale: float, chunk: int = 0) -> torch.Tensor:
     """The recurrence S <- diag(exp(log_decay_t)) S + k_t v_t^T, o_t = S^T q_t qscale, for every sequence of the step from
-    its state slot (``state`` float32 [slots, heads, dk, dv], updated in place).  Returns o float32 [T, heads * dv]."""
+    its state slot (``state`` float32 [slots, heads, dk, dv], updated in place).  Returns o float32 [T, heads * dv].
+    ``chunk`` > 0: sequences are cut into chunks of that many tokens that run side by side (every chunk from zero, a walk
+    over the chunks' states, every chunk again from its true state): the same sums in another order."""
     _gpu(x, log_decay, cu_seqlens, state_slots, state)
     T = x.shape[0]
     if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < max(q_col + heads * dk, k_col + heads * dk, v_col + heads * dv):
@@ -700,10 +733,16 @@ def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: tor
     _i32(cu_seqlens, "cu_seqlens", num_seqs + 1)
     _i32(state_slots, "state_slots", num_seqs)
     out = torch.empty(T, heads * dv, dtype=torch.float32, device=x.device)
+    ws = ws_decay = None
+    max_chunks = 0
+    if chunk > 0:
+        max_chunks = -(-T // chunk)
+        ws = torch.empty(num_seqs * max_chunks, heads, dk, dv, dtype=torch.float32, device=x.device)
+        ws_decay = torch.empty(num_seqs * max_chunks, heads, dk, dtype=torch.float32, device=x.device)
     lib = library.core()
     _check(lib, lib.pico_gla_scan(_ptr(x), x.stride(0) if T > 1 else x.shape[1], _dt(x), q_col, k_col, v_col, _ptr(log_decay),
                                   _ptr(cu_seqlens), _ptr(state_slots), _ptr(state), _ptr(out), num_seqs, T, heads, dk, dv,
-                                  c_float(qscale), state.shape[0], _stream()))
+                                  c_float(qscale), state.shape[0], chunk, max_chunks, _ptr(ws), _ptr(ws_decay), _stream()))
     return out
 
 

@@ -113,6 +113,10 @@ class GatedAttention(Mixer):
     def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
         return self.o.partial(self.attend(x, ctx, cache))
 
+    def forward_into(self, x: torch.Tensor, ctx: StepContext, cache, resid: torch.Tensor) -> None:
+        """resid += the mixer's output: with few rows the sum is the epilogue of the output projection."""
+        self.o.add_into(self.attend(x, ctx, cache), resid)
+
     def attend(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
         """The gated heads' outputs [T, H dv] in front of the output projection."""
         reads_other = bool(getattr(cache, "read_only", False))

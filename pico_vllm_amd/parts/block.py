@@ -71,8 +71,10 @@ class ParallelBlock(Block):
 @register_part("block", "parallel_two_norms")
 class ParallelTwoNormBlock(Block):
     """x += mixer(norm1(x)) + ff(norm2(x)): both sublayers read the same x, each through a norm of its own.  The sums
-    are float32.  A delta that is still pending joins the stream in the first norm's launch; the second norm then reads
-    the summed stream.  The mixer's output joins the stream at once, the feed-forward's last delta is handed on as
+    are float32.  A delta that is still pending joins the stream in the norms' launch (one launch makes both norms where
+    they differ in their weights only).  The mixer's output joins the stream at once (a mixer with
+    ``forward_into(h, ctx, cache, resid)`` adds it itself, as the last step of its output projection); so does what a
+    feed-forward with ``forward_into(h, ctx, resid)`` adds itself; the feed-forward's last delta is handed on as
     ``pending`` (a feed-forward may return a list of deltas: all but the last are added here).  A layer without a
     feed-forward names the part "none" in that slot."""
     slot_categories = {"norm1": "norm", "mixer": "mixer", "norm2": "norm", "ff": "feed_forward"}
@@ -85,13 +87,21 @@ class ParallelTwoNormBlock(Block):
 
     def forward(self, resid, pending, ctx, cache):
         p = self.parts
-        h1 = p["norm1"].add_norm(resid, pending)
-        h2 = p["norm2"].add_norm(resid, None)
-        a = p["mixer"].forward(h1, ctx, cache)
-        f = p["ff"].forward(h2, ctx)
-        if f is None:
-            return resid, a
-        self._add(resid, a)
+        if pending is not None and pending.dim() == 3 and pending.shape[0] > kernels.MAX_SLABS:
+            self._add(resid, pending)                          # more partial sums than a norm's launch takes
+            pending = None
+        pair = getattr(p["norm1"], "add_norm_pair", None)
+        both = pair(p["norm2"], resid, pending) if pair is not None else None
+        if both is None:
+            both = (p["norm1"].add_norm(resid, pending), p["norm2"].add_norm(resid, None))
+        h1, h2 = both
+        into = getattr(p["mixer"], "forward_into", None)
+        if into is not None:
+            into(h1, ctx, cache, resid)
+        else:
+            self._add(resid, p["mixer"].forward(h1, ctx, cache))
+        into = getattr(p["ff"], "forward_into", None)
+        f = into(h2, ctx, resid) if into is not None else p["ff"].forward(h2, ctx)
         if isinstance(f, (list, tuple)):
             for d in f[:-1]:
                 self._add(resid, d)

@@ -28,6 +28,11 @@ class GatedLinearAttention(Mixer):
 
     graph_safe_prompts = True
 
+    # In the bfloat16 engine a step with a prompt portion cuts its sequences into chunks of this many tokens that run
+    # side by side (``kernels.gla_scan``); decided from the step's shape alone.  The 32-bit engine walks every sequence
+    # whole, so that its sums do not depend on how a prompt was cut.
+    CHUNK, CHUNKED_FROM = 64, 128
+
     NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm", "a1": "a1", "a2": "a2", "a2_bias": "a2.b"}
 
     def __init__(self, hidden_size: int, num_heads: int, key_dim: int, value_dim: int, tau: float, rank: int, norm_eps: float,
@@ -77,9 +82,17 @@ class GatedLinearAttention(Mixer):
         return super().weight_bytes() + self.a2.numel() * self.a2.element_size()
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
+        return self.o.partial(self.mix(x, ctx, cache))
+
+    def forward_into(self, x: torch.Tensor, ctx: StepContext, cache, resid: torch.Tensor) -> None:
+        """resid += the mixer's output: with few rows the sum is the epilogue of the output projection."""
+        self.o.add_into(self.mix(x, ctx, cache), resid)
+
+    def mix(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
+        """The normed and gated heads' outputs [T, H dv] in front of the output projection."""
         y = self.proj(x)                                   # [T, q | k | v | g | a1]
         log_decay = kernels.gla_decay(y, self.a_col, self.a2, self.a2_bias, self.tau)
+        chunked = self.act_dtype == torch.bfloat16 and not ctx.all_decode and ctx.num_tokens >= self.CHUNKED_FROM
         o = kernels.gla_scan(y, self.q_col, self.k_col, self.v_col, log_decay, ctx.cu_seqlens, ctx.state_slots, cache.state,
-                             ctx.num_seqs, self.heads, self.dk, self.dv, self.dk ** -0.5)
-        a = kernels.gla_out(o, y, self.g_col, self.norm_weight, self.norm_eps, self.heads, self.dv)
-        return self.o.partial(a)
+                             ctx.num_seqs, self.heads, self.dk, self.dv, self.dk ** -0.5, chunk=self.CHUNK if chunked else 0)
+        return kernels.gla_out(o, y, self.g_col, self.norm_weight, self.norm_eps, self.heads, self.dv)

@@ -161,6 +161,19 @@ class SoftmaxRoutedExperts(FeedForward):
         return 2.0 * tokens * (self.outputs * D + self.top * 3 * F * D) + (self.shared.flops(tokens, pairs) if self.shared is not None else 0.0)
 
     def forward(self, x: torch.Tensor, ctx: StepContext):
+        out = self._routed(x)
+        if self.shared is None:
+            return out
+        return [self.shared.forward(x, ctx), out]
+
+    def forward_into(self, x: torch.Tensor, ctx: StepContext, resid: torch.Tensor):
+        """The shared expert's second product adds into the float32 stream ``resid`` itself (its epilogue in a small
+        step); the routed sum is returned, for the next norm's launch to add."""
+        if self.shared is not None:
+            self.shared.down.add_into(self.shared.gate_up.swiglu(x), resid)
+        return self._routed(x)
+
+    def _routed(self, x: torch.Tensor) -> torch.Tensor:
         E, F, D = self.num_experts, self.expert_size, self.hidden_size
         experts, weights = kernels.moe_router_softmax(x, self.router.weight, self.correction, self.top, self.scale)
         gate_up = self.gate_up.weight.view(E, 2 * F, D)
@@ -172,9 +185,7 @@ class SoftmaxRoutedExperts(FeedForward):
             out = kernels.moe_experts_plain(xe, gate_up, down, experts, weights, 0.0, 0.0, mode=kernels.MOE_SWIGLU)
         if self.identity:
             kernels.moe_identity(xe, experts, weights, out, E)
-        if self.shared is None:
-            return out
-        return [out, self.shared.forward(x, ctx)]
+        return out
 
     def graph_variant(self, ctx: StepContext) -> tuple:
         return (("softmax_routed_experts", kernels.moe_grouped_rows(ctx.num_tokens, self.top)),)

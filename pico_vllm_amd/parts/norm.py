@@ -30,6 +30,12 @@ class RMSNorm(Norm):
     def add_norm(self, resid, delta, rows=None):
         return kernels.add_rmsnorm(resid, delta, self.weight, self.eps, self.act_dtype, rows)
 
+    def add_norm_pair(self, other: "RMSNorm", resid, delta):
+        """(this norm, ``other``) of resid + delta in one launch where the two differ in their weights only; else None."""
+        if not isinstance(other, RMSNorm) or (other.size, other.eps, other.act_dtype) != (self.size, self.eps, self.act_dtype):
+            return None
+        return kernels.add_rmsnorm2(resid, delta, self.weight, other.weight, self.eps, self.act_dtype)
+
     def deferred(self, resid, delta):
         # the one row of a bfloat16 step: the projection behind the norm can norm it itself
         if (self.act_dtype == torch.bfloat16 and resid.shape[0] <= kernels.SKINNY_NORM_ROWS

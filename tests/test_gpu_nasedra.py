@@ -380,6 +380,27 @@ def test_gla_kernels_in_portions_and_token_by_token(dtype, H, dk, dv, rank, tau)
             whole = got
         elif dtype == "float32":
             assert torch.equal(got, whole)     # the same bits however the sequences were cut
+    # sequences cut into chunks that run side by side: the same sums in another order
+    cu = torch.tensor(np.cumsum([0] + lens), dtype=torch.int32, device=DEV)
+    sl = torch.tensor(slots_of, dtype=torch.int32, device=DEV)
+    for chunk in (4, 16, 64):
+        state = torch.full((5, H, dk, dv), 3.0, device=DEV)
+        for s_ in slots_of:
+            state[s_] = 0
+        half = [n // 2 for n in lens]           # first the front halves (from the slots' zeros), then the rest from the state
+        for part in (0, 1):
+            rows = torch.cat([torch.arange(sum(lens[:bi]) + (0 if part == 0 else half[bi]), sum(lens[:bi]) + (half[bi] if part == 0 else n))
+                              for bi, n in enumerate(lens)])
+            counts = [half[bi] if part == 0 else n - half[bi] for bi, n in enumerate(lens)]
+            keep = [bi for bi, c in enumerate(counts) if c > 0]
+            cu_p = torch.tensor(np.cumsum([0] + [counts[bi] for bi in keep]), dtype=torch.int32, device=DEV)
+            sl_p = torch.tensor([slots_of[bi] for bi in keep], dtype=torch.int32, device=DEV)
+            o = K.gla_scan(xd[rows.to(DEV)].contiguous(), 0, offs[1], offs[2], ld[rows.to(DEV)].contiguous(), cu_p, sl_p, state,
+                           len(keep), H, dk, dv, dk ** -0.5, chunk=chunk)
+            assert torch.allclose(o.cpu().double(), want_o.view(T, -1)[rows], **tol), (chunk, part)
+        for bi, s_ in enumerate(slots_of):
+            assert torch.allclose(state[s_].cpu().double(), want_S[bi], **tol), (chunk, bi)
+        assert bool((state[1] == 3.0).all()) and bool((state[4] == 3.0).all())
     out = K.gla_out(torch.cat(outs).to(DEV), xd, offs[3], w.to(DEV), eps, H, dv)
     ref = (P.rms_norm(torch.cat(outs).double().view(T, H, dv), w.double(), eps).reshape(T, H * dv) * P.silu(gate))
     assert torch.allclose(out.cpu().double(), ref, rtol=1e-5 if dtype == "float32" else 1e-2, atol=1e-5 if dtype == "float32" else 1e-2)
