@@ -52,9 +52,9 @@ extern "C" int pico_gla_decay(const void* x, int ldx, int dtype, const void* a2,
 // ---------------------------------------------------------------------------
 // The recurrence, token by token.  grid (sequences, heads, ceil(dv / 64)); a workgroup owns 64 value channels of one
 // head of one sequence; wave w of its ceil(dk / GLA_CPT) waves owns key channels GLA_CPT w .., lane l value channel l:
-// a thread keeps GLA_CPT state elements in registers over all tokens of the step.  Tokens are taken GLA_TB at a time:
-// their q, k and decays are staged in LDS (every thread reads all of its channels' from there), the waves' partial
-// outputs meet in LDS and are summed in wave order.
+// a thread keeps GLA_CPT state elements in registers over all tokens of the step.  Tokens are taken TB (8 or 16) at a
+// time: their q, k and decays are staged in LDS (every thread reads all of its channels' from there) while the next
+// block's travel from memory in registers; the waves' partial outputs meet in LDS and are summed in wave order.
 //
 // Long portions are cut into chunks of `chunk` tokens that run side by side (the recurrence is linear in the state):
 //   GLA_LOCAL:  every chunk from a state of zero, no outputs; leaves its state in ws[chunk] and the sum of its decays'
@@ -64,26 +64,26 @@ extern "C" int pico_gla_decay(const void* x, int ldx, int dtype, const void* a2,
 // GLA_WHOLE is the plain walk from the slot's state (a sequence is one chunk).  blockIdx.x = sequence * max_chunks + chunk.
 // ---------------------------------------------------------------------------
 #define GLA_CPT 32
-#define GLA_TB 8
 #define GLA_WHOLE 0
 #define GLA_LOCAL 1
 #define GLA_FROM 2
 
-template <typename T, int MODE>
+template <typename T, int MODE, int TB>
 __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, int ldx, int q_col, int k_col, int v_col,
                                                        const float* __restrict__ log_decay,
                                                        const int* __restrict__ cu_seqlens,
                                                        const int* __restrict__ state_slots, float* __restrict__ state,
                                                        float* __restrict__ out, int H, int dk, int dv, float qscale,
                                                        int num_slots, int chunk, int max_chunks, float* __restrict__ ws,
-                                                       float* __restrict__ ws_decay) {
+                                                       float* __restrict__ ws_decay, const T* __restrict__ a2,
+                                                       const float* __restrict__ a2_bias, int a_col, int R, float inv_tau) {
   extern __shared__ float lds[];
   const int nw = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int CP = nw * GLA_CPT;                          // key channels with padding
-  float* qs = lds;                                      // [GLA_TB][CP]
-  float* ks = qs + GLA_TB * CP;
-  float* as = ks + GLA_TB * CP;
-  float* po = as + GLA_TB * CP;                         // [GLA_TB][nw][64]
+  float* qs = lds;                                      // [TB][CP]
+  float* ks = qs + TB * CP;
+  float* as = ks + TB * CP;
+  float* po = as + TB * CP;                             // [TB][nw][64]
   const int b = MODE == GLA_WHOLE ? blockIdx.x : blockIdx.x / max_chunks, h = blockIdx.y, v = blockIdx.z * 64 + lane;
   const bool v_ok = v < dv;
   int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1];
@@ -107,28 +107,56 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
       ws_decay[((size_t)blockIdx.x * H + h) * dk + c] = sum;
     }
   }
-
-  for (int t0 = t_begin; t0 < t_end; t0 += GLA_TB) {
-    const int nb = min(GLA_TB, t_end - t0);
-    __syncthreads();                                    // the last block's partial outputs have been read
-    for (int i = threadIdx.x; i < nb * CP; i += blockDim.x) {
-      const int tt = i / CP, c = i - tt * CP;
+  // A thread stages TB / 2 elements (token tt, channel c) of a block: i = threadIdx.x + j * blockDim.x.  The next
+  // block's values travel in registers while this block is walked.
+  constexpr int NL = TB / 2;
+  float rq[NL], rk[NL], ra[NL], rv[TB];
+  auto fetch = [&](int t0) {
+    const int nb = min(TB, t_end - t0);
+#pragma unroll
+    for (int j = 0; j < NL; j++) {
+      const int i = threadIdx.x + j * blockDim.x, tt = i / CP, c = i - tt * CP;
       float qv = 0.f, kv = 0.f, av = 1.f;
-      if (c < dk) {
+      if (tt < nb && c < dk) {
         const T* row = x + (size_t)(t0 + tt) * ldx + (size_t)h * dk + c;
         if (MODE != GLA_LOCAL) qv = load_f32(row + q_col) * qscale;
         kv = load_f32(row + k_col);
-        av = expf(log_decay[(size_t)(t0 + tt) * H * dk + (size_t)h * dk + c]);
+        if (log_decay) {
+          av = log_decay[(size_t)(t0 + tt) * H * dk + (size_t)h * dk + c];
+        } else {
+          // the decay's logarithm made here from the low-rank activations (as gla_decay_kernel does): one launch less
+          const T* xa = x + (size_t)(t0 + tt) * ldx + a_col;
+          const T* w = a2 + ((size_t)h * dk + c) * R;
+          float z = a2_bias ? a2_bias[h * dk + c] : 0.f;
+          for (int r = 0; r < R; r++) z = fmaf(load_f32(w + r), load_f32(xa + r), z);
+          const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+          av = ls * inv_tau;
+        }
       }
-      qs[i] = qv; ks[i] = kv; as[i] = av;
+      rq[j] = qv; rk[j] = kv; ra[j] = av;
     }
-    float vv[GLA_TB];
 #pragma unroll
-    for (int tt = 0; tt < GLA_TB; tt++)
-      vv[tt] = (tt < nb && v_ok) ? load_f32(x + (size_t)(t0 + tt) * ldx + v_col + (size_t)h * dv + v) : 0.f;
+    for (int tt = 0; tt < TB; tt++)
+      rv[tt] = (tt < nb && v_ok) ? load_f32(x + (size_t)(t0 + tt) * ldx + v_col + (size_t)h * dv + v) : 0.f;
+  };
+  fetch(t_begin);
+  for (int t0 = t_begin; t0 < t_end; t0 += TB) {
+    const int nb = min(TB, t_end - t0);
+    __syncthreads();                                    // the last block's staged values and partial outputs have been read
+#pragma unroll
+    for (int j = 0; j < NL; j++) {
+      const int i = threadIdx.x + j * blockDim.x, tt = i / CP, c = i - tt * CP;
+      qs[i] = rq[j];
+      ks[i] = rk[j];
+      as[i] = (tt < nb && c < dk) ? expf(ra[j]) : 1.f;
+    }
+    float vv[TB];
+#pragma unroll
+    for (int tt = 0; tt < TB; tt++) vv[tt] = rv[tt];
     __syncthreads();
+    if (t0 + TB < t_end) fetch(t0 + TB);
 #pragma unroll
-    for (int tt = 0; tt < GLA_TB; tt++) {
+    for (int tt = 0; tt < TB; tt++) {
       if (tt >= nb) break;
       const float4* a4 = reinterpret_cast<const float4*>(as + tt * CP + c0);
       const float4* k4 = reinterpret_cast<const float4*>(ks + tt * CP + c0);
@@ -192,13 +220,18 @@ __global__ __launch_bounds__(256) void gla_combine_kernel(const int* __restrict_
   *sp = S;
 }
 
+// log_decay null (chunk == 0 only): the decays are made inside the walk from x[:, a_col : a_col + R], a2 [H dk, R] and
+// a2_bias, as pico_gla_decay makes them.
 // chunk == 0: every sequence walked whole from its slot.  chunk > 0: sequences cut into chunks of that many tokens that
 // run side by side (three launches); ws float32 [num_seqs * max_chunks, H, dk, dv], ws_decay [num_seqs * max_chunks, H, dk],
 // max_chunks at least the chunks of the longest sequence.
 extern "C" int pico_gla_scan(const void* x, int ldx, int dtype, int q_col, int k_col, int v_col, const float* log_decay,
                              const int* cu_seqlens, const int* state_slots, float* state, float* out, int num_seqs,
                              int T, int H, int dk, int dv, float qscale, int num_slots, int chunk, int max_chunks,
-                             float* ws, float* ws_decay, hipStream_t stream) {
+                             float* ws, float* ws_decay, const void* a2, const float* a2_bias, int a_col, int R, float tau,
+                             hipStream_t stream) {
+  PICO_REQUIRE(log_decay != nullptr || (chunk == 0 && a2 != nullptr && R > 0 && a_col >= 0 && ldx >= a_col + R && tau > 0.f),
+               "pico_gla_scan: without the decays' logarithms the walk needs what makes them, and runs whole");
   PICO_REQUIRE(num_seqs >= 0 && T >= 0 && H > 0 && dk > 0 && dv > 0 && num_slots > 0, "pico_gla_scan: bad sizes");
   PICO_REQUIRE(dk <= 8 * GLA_CPT, "pico_gla_scan: at most %d key channels a head, got %d", 8 * GLA_CPT, dk);
   PICO_REQUIRE(q_col >= 0 && k_col >= 0 && v_col >= 0 && ldx >= q_col + H * dk && ldx >= k_col + H * dk && ldx >= v_col + H * dv,
@@ -209,13 +242,21 @@ extern "C" int pico_gla_scan(const void* x, int ldx, int dtype, int q_col, int k
                "pico_gla_scan: chunks need room for their states and must cover the step's tokens");
   if (num_seqs == 0 || T == 0) return 0;
   const int nw = (dk + GLA_CPT - 1) / GLA_CPT;
-  const size_t lds = (size_t)(3 * GLA_TB * nw * GLA_CPT + GLA_TB * nw * 64) * sizeof(float);
+  // tokens of a block: 16 where the staged values fit (up to 128 key channels), else 8
+  const int tb = nw <= 4 ? 16 : 8;
+  const size_t lds = (size_t)(3 * tb * nw * GLA_CPT + tb * nw * 64) * sizeof(float);
   PICO_REQUIRE(lds <= 64 * 1024, "pico_gla_scan: key channels beyond the staging memory");
   const int vb = (dv + 63) / 64;
-#define GLA_LAUNCH(TT, MODE, GX)                                                                                          \
-  gla_scan_kernel<TT, MODE><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>((const TT*)x, ldx, q_col, k_col, v_col, log_decay,    \
-                                                                      cu_seqlens, state_slots, state, out, H, dk, dv, qscale, \
-                                                                      num_slots, chunk, max_chunks, ws, ws_decay)
+#define GLA_ARGS(TT)                                                                                                       \
+  (const TT*)x, ldx, q_col, k_col, v_col, log_decay, cu_seqlens, state_slots, state, out, H, dk, dv, qscale, num_slots,   \
+      chunk, max_chunks, ws, ws_decay, (const TT*)a2, a2_bias, a_col, R, 1.0f / (tau > 0.f ? tau : 1.f)
+#define GLA_LAUNCH(TT, MODE, GX)                                                                                           \
+  do {                                                                                                                     \
+    if (tb == 16)                                                                                                          \
+      gla_scan_kernel<TT, MODE, 16><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                              \
+    else                                                                                                                   \
+      gla_scan_kernel<TT, MODE, 8><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                               \
+  } while (0)
 #define GLA_RUN(TT)                                                                                                        \
   if (chunk == 0) {                                                                                                        \
     GLA_LAUNCH(TT, GLA_WHOLE, num_seqs);                                                                                   \
@@ -235,6 +276,7 @@ extern "C" int pico_gla_scan(const void* x, int ldx, int dtype, int q_col, int k
   }
 #undef GLA_RUN
 #undef GLA_LAUNCH
+#undef GLA_ARGS
   PICO_LAUNCH_CHECK();
   return 0;
 }

@@ -146,7 +146,7 @@ static int moe_router_impl(const void* x, int ldx, int dtype, const float* Wr, i
   else { if (vec) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
 #undef LAUNCH
   if (softmax)
-    moe_route_softmax_kernel<<<(T + 63) / 64, 64, 0, stream>>>(z, correction, T, E, top, scale, experts, weights);
+    moe_route_softmax_kernel<<<(T + 3) / 4, 256, 0, stream>>>(z, correction, T, E, top, scale, experts, weights);
   else
     moe_route_kernel<<<(T + 63) / 64, 64, 0, stream>>>(z, T, E, top, experts, weights);
   PICO_LAUNCH_CHECK();
@@ -175,43 +175,49 @@ __device__ __forceinline__ float expert_act(float g, float u, float limit, float
 }
 
 // ---------------------------------------------------------------------------
-// Choice by softmax scores with a correction: one thread per token.  z [T, E] float32 router logits (E counts every
-// router output); correction [E] or null.
+// Choice by softmax scores with a correction: one wave per token, lane l looks after router outputs l, l + 64, ...
+// z [T, E] float32 router logits (E counts every router output); correction [E] or null.  Sums and maxima run over the
+// wave in a fixed order; among equal choice scores the lowest output wins.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void moe_route_softmax_kernel(const float* __restrict__ logits,
-                                                               const float* __restrict__ correction, int T, int E, int top,
-                                                               float scale, int* __restrict__ experts,
-                                                               float* __restrict__ weights) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(256) void moe_route_softmax_kernel(const float* __restrict__ logits,
+                                                                const float* __restrict__ correction, int T, int E, int top,
+                                                                float scale, int* __restrict__ experts,
+                                                                float* __restrict__ weights) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (t >= T) return;
   const float* z = logits + (size_t)t * E;
-  float mx = z[0];
-  for (int e = 1; e < E; e++) mx = fmaxf(mx, z[e]);
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+  mx = wave_max(mx);
   float den = 0.f;
-  for (int e = 0; e < E; e++) den += expf(z[e] - mx);
-  const float inv = 1.0f / den;
+  for (int e = lane; e < E; e += 64) den += expf(z[e] - mx);
+  const float inv = 1.0f / wave_sum(den);
   int chosen[MOE_MAX_TOP];
   float score[MOE_MAX_TOP];
   float total = 0.f;
   for (int k = 0; k < top; k++) {
-    int best = -1;
-    float bc = 0.f, bs = 0.f;
-    for (int e = 0; e < E; e++) {
+    float bc = -INFINITY;
+    int best = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
       bool taken = false;
       for (int j = 0; j < k; j++) taken |= chosen[j] == e;
       if (taken) continue;
-      const float sc = expf(z[e] - mx) * inv;
-      const float c = sc + (correction ? correction[e] : 0.f);
-      if (best < 0 || c > bc) { best = e; bc = c; bs = sc; }
+      const float c = expf(z[e] - mx) * inv + (correction ? correction[e] : 0.f);
+      if (c > bc || best == 0x7fffffff) { best = e; bc = c; }     // a lane's outputs come in ascending order: the first of equals stays
     }
+    wave_first_max(bc, best);
     chosen[k] = best;
-    score[k] = bs;
-    total += bs;
+    score[k] = expf(z[min(best, E - 1)] - mx) * inv;
+    total += score[k];
   }
   const float f = scale / (total + 1e-20f);
-  for (int k = 0; k < top; k++) {
-    experts[(size_t)t * top + k] = chosen[k];
-    weights[(size_t)t * top + k] = score[k] * f;
+  if (lane < top) {
+    // (chosen and score are the same in every lane)
+    for (int k = 0; k < top; k++)
+      if (k == lane) {
+        experts[(size_t)t * top + k] = chosen[k];
+        weights[(size_t)t * top + k] = score[k] * f;
+      }
   }
 }
 

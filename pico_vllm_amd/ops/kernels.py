@@ -713,18 +713,31 @@ def gla_decay(x: torch.Tensor, col: int, a2: torch.Tensor, bias: Optional[torch.
 GLA_MAX_KEY_DIM = 256
 
 
-def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: torch.Tensor, cu_seqlens: torch.Tensor,
+def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: Optional[torch.Tensor], cu_seqlens: torch.Tensor,
              state_slots: torch.Tensor, state: torch.Tensor, num_seqs: int, heads: int, dk: int, dv: int,
-             qscale: float, chunk: int = 0) -> torch.Tensor:
+             qscale: float, chunk: int = 0, decay_from: Optional[tuple] = None) -> torch.Tensor:
     """The recurrence S <- diag(exp(log_decay_t)) S + k_t v_t^T, o_t = S^T q_t qscale, for every sequence of the step from
     its state slot (``state`` float32 [slots, heads, dk, dv], updated in place).  Returns o float32 [T, heads * dv].
     ``chunk`` > 0: sequences are cut into chunks of that many tokens that run side by side (every chunk from zero, a walk
-    over the chunks' states, every chunk again from its true state): the same sums in another order."""
+    over the chunks' states, every chunk again from its true state): the same sums in another order.
+    ``log_decay`` None (whole walks only): the decays are made inside the launch from ``decay_from`` = (column of the
+    low-rank activations in x, a2 [heads * dk, R], bias float32 or None, tau), as ``gla_decay`` makes them."""
     _gpu(x, log_decay, cu_seqlens, state_slots, state)
     T = x.shape[0]
     if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < max(q_col + heads * dk, k_col + heads * dk, v_col + heads * dv):
         raise KernelError("gla_scan: x must be [T, columns] with unit stride along the row and hold q, k and v")
-    if log_decay.dtype != torch.float32 or tuple(log_decay.shape) != (T, heads * dk) or not log_decay.is_contiguous():
+    a_col, a2, a2_bias, tau, R = 0, None, None, 0.0, 0
+    if log_decay is None:
+        if chunk or decay_from is None:
+            raise KernelError("gla_scan: without the decays' logarithms the walk runs whole and needs what makes them")
+        a_col, a2, a2_bias, tau = decay_from
+        _gpu(a2, a2_bias)
+        R = a2.shape[1]
+        if a2.dtype != x.dtype or tuple(a2.shape) != (heads * dk, R) or not a2.is_contiguous() or x.shape[1] < a_col + R:
+            raise KernelError("gla_scan: a2 [heads * dk, R] of x's dtype, and x must hold the R low-rank activations")
+        if a2_bias is not None and (a2_bias.dtype != torch.float32 or a2_bias.shape != (heads * dk,) or not a2_bias.is_contiguous()):
+            raise KernelError("gla_scan: the decay's bias must be contiguous float32")
+    elif log_decay.dtype != torch.float32 or tuple(log_decay.shape) != (T, heads * dk) or not log_decay.is_contiguous():
         raise KernelError(f"gla_scan: the decays' logarithms must be contiguous float32 [{T}, {heads * dk}]")
     if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dk, dv) or not state.is_contiguous():
         raise KernelError(f"gla_scan: the state must be contiguous float32 [slots, {heads}, {dk}, {dv}]")
@@ -742,7 +755,8 @@ def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: tor
     lib = library.core()
     _check(lib, lib.pico_gla_scan(_ptr(x), x.stride(0) if T > 1 else x.shape[1], _dt(x), q_col, k_col, v_col, _ptr(log_decay),
                                   _ptr(cu_seqlens), _ptr(state_slots), _ptr(state), _ptr(out), num_seqs, T, heads, dk, dv,
-                                  c_float(qscale), state.shape[0], chunk, max_chunks, _ptr(ws), _ptr(ws_decay), _stream()))
+                                  c_float(qscale), state.shape[0], chunk, max_chunks, _ptr(ws), _ptr(ws_decay), _ptr(a2),
+                                  _ptr(a2_bias), a_col, R, c_float(tau), _stream()))
     return out
 
 

@@ -91,8 +91,10 @@ class GatedLinearAttention(Mixer):
     def mix(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
         """The normed and gated heads' outputs [T, H dv] in front of the output projection."""
         y = self.proj(x)                                   # [T, q | k | v | g | a1]
-        log_decay = kernels.gla_decay(y, self.a_col, self.a2, self.a2_bias, self.tau)
         chunked = self.act_dtype == torch.bfloat16 and not ctx.all_decode and ctx.num_tokens >= self.CHUNKED_FROM
+        # a whole walk makes its decays itself (the same arithmetic, one launch less); chunks need them beforehand
+        log_decay = kernels.gla_decay(y, self.a_col, self.a2, self.a2_bias, self.tau) if chunked else None
         o = kernels.gla_scan(y, self.q_col, self.k_col, self.v_col, log_decay, ctx.cu_seqlens, ctx.state_slots, cache.state,
-                             ctx.num_seqs, self.heads, self.dk, self.dv, self.dk ** -0.5, chunk=self.CHUNK if chunked else 0)
+                             ctx.num_seqs, self.heads, self.dk, self.dv, self.dk ** -0.5, chunk=self.CHUNK if chunked else 0,
+                             decay_from=(self.a_col, self.a2, self.a2_bias, self.tau))
         return kernels.gla_out(o, y, self.g_col, self.norm_weight, self.norm_eps, self.heads, self.dv)

@@ -365,7 +365,11 @@ def test_gla_kernels_in_portions_and_token_by_token(dtype, H, dk, dv, rank, tau)
             cu = torch.tensor(np.cumsum([0] + [m for _, _, m in step]), dtype=torch.int32, device=DEV)
             sl = torch.tensor([slots_of[bi] for bi, _, _ in step], dtype=torch.int32, device=DEV)
             xs = xd[rows.to(DEV)].contiguous()
-            o = K.gla_scan(xs, 0, offs[1], offs[2], ld[rows.to(DEV)].contiguous(), cu, sl, state, len(step), H, dk, dv, dk ** -0.5)
+            if parts is None:                  # token by token: the decays made inside the walk
+                o = K.gla_scan(xs, 0, offs[1], offs[2], None, cu, sl, state, len(step), H, dk, dv, dk ** -0.5,
+                               decay_from=(offs[4], a2.to(DEV), b.to(DEV), tau))
+            else:
+                o = K.gla_scan(xs, 0, offs[1], offs[2], ld[rows.to(DEV)].contiguous(), cu, sl, state, len(step), H, dk, dv, dk ** -0.5)
             a = 0
             for bi, d, m in step:
                 outs[bi][d:d + m] = o[a:a + m].cpu()
