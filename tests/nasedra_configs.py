@@ -84,6 +84,12 @@ CONFIGS = {
         (gla(1, 80, 100, 1.0), None),
         (attention(2, 1, 64, 16, 33, 2, None, None, scale=0.2), dense(64)),
         (gla(3, 16, 8, 30.0), moe(8, 4, 24, identity=3, scale=2.0, shared=16))]), 3),
+    # a width that is no multiple of 8, a vocabulary that is odd, two heads on two kv heads, a window of one page with
+    # more kept positions than a page holds, every router output chosen
+    "d": (config(51, 44, [
+        (gla(2, 12, 20, 2.0), dense(36)),
+        (attention(2, 2, 12, 20, 16, 18, 25.0, rot(6, 200.0, (2.0, 16, 4.0, 1.0)), scale=0.31), moe(2, 3, 20, identity=1, scale=1.2, shared=12)),
+        (attention(2, 2, 12, 20, 7, 0, None, rot(6, 200.0, (2.0, 16, 4.0, 1.0)), kv_from=1), dense(28))], eps=1e-6, embed_scale=2.5), 4),
 }
 
 

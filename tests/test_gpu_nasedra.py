@@ -494,7 +494,7 @@ def test_experts_with_pass_through_outputs_and_a_shared_expert(dtype, E, ident, 
 # ---------------------------------------------------------------------------------------------------------------
 # whole models through the replayer
 # ---------------------------------------------------------------------------------------------------------------
-PAGE = {"a": 16, "b": 8, "c": 32}
+PAGE = {"a": 16, "b": 8, "c": 32, "d": 16}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
