@@ -24,7 +24,7 @@ from .lerazen import _int, _num
 from .model_config import ConfigError
 from .registry import register_architecture
 
-DEFAULT_DECAY_RANK = 16      # where neither a checkpoint nor the configuration says (a model yet to be written)
+DEFAULT_DECAY_RANK = 32      # where neither a checkpoint nor the configuration says (a model yet to be written)
 
 
 @dataclass(frozen=True)

@@ -54,17 +54,17 @@ def _nasedra(vocab, width, layers, heads, kv_heads, dim, dense_ff, experts, top,
     """A Nasedra configuration of a real model's proportions, in groups of four layers: windowed attention with a dense
     feed-forward, a recurrent layer with a routed one, attention over the first layer's keys and values with a dense
     one, a recurrent layer with a routed one."""
-    rot = {"dims": dim, "base": 500000.0, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+    rot = {"dims": dim, "base": 1000000.0, "scaling": {"factor": 4.0, "original": 8192, "fast": 16.0, "slow": 2.0}}
 
     def attention(i):
-        m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 50.0,
+        m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 30.0,
              "mask": {"size": window, "keep_first": keep_first}, "rot": rot}
         if i % 4 == 2:
             m["kv_from"] = i - 2
         return m
-    recurrent = {"heads": heads, "dim": gla_dim, "vdim": dim, "tau": 16.0}
+    recurrent = {"heads": heads, "dim": gla_dim, "vdim": dim, "tau": 8.0, "rank": 32}
     dense = {"kind": "dense", "ff": dense_ff}
-    routed = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "identity": 2, "scale": 1.5},
+    routed = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "identity": 1, "scale": 2.0},
               "shared": {"ff": shared_ff}}
     return {"architecture": "Nasedra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": width ** 0.5},
             "layers": [{"type": "gla", "mixer": recurrent, "mlp": routed} if i % 2 else

@@ -66,17 +66,17 @@ CONFIGS = {
     # values through another mask, experts with two pass-through outputs and a shared expert
     "a": (config(97, 72, [
         (attention(3, 1, 24, 40, 12, 3, 30.0, rot(16, 10000.0, YARN)), dense(100)),
-        (gla(2, 24, 40, 4.0), moe(5, 2, 32, identity=2, scale=1.5, shared=48)),
+        (gla(2, 24, 40, 4.0), moe(5, 2, 32, identity=2, scale=1.25, shared=48)),
         (attention(3, 1, 24, 40, 20, 1, 30.0, rot(16, 10000.0, YARN), kv_from=0), dense(100)),
         (gla(2, 24, 40, 4.0), dense(64))], embed_scale=3.0), 5),
     # sizes the matrix-core kernels take: a window that spans pages with kept positions, a recurrent layer first, several
     # kv heads, the whole head rotated without scaling, three of seven router outputs, no cap on one layer, layers that
     # differ in their heads
     "b": (config(256, 128, [
-        (gla(4, 64, 64, 16.0), moe(6, 3, 64, identity=1)),
-        (attention(8, 2, 64, 32, 44, 5, None, rot(64, 500000.0)), dense(256)),
+        (gla(4, 64, 64, 12.0), moe(6, 3, 64, identity=1)),
+        (attention(8, 2, 64, 32, 44, 5, None, rot(64, 300000.0)), dense(256)),
         (attention(4, 4, 32, 64, 100, 20, 15.0, rot(32, 1000.0, (8.0, 32, 4.0, 0.5))), moe(4, 1, 32, identity=2, scale=0.7, shared=64)),
-        (attention(8, 2, 64, 32, 17, 0, 8.0, rot(64, 500000.0), kv_from=1), None)], eps=1e-6), 16),
+        (attention(8, 2, 64, 32, 17, 0, 8.0, rot(64, 300000.0), kv_from=1), None)], eps=1e-6), 16),
     # no mask at all, as many kv heads as heads, no rotation on one layer, a recurrent layer whose key channels fill three
     # waves and whose values two workgroups, one expert a token, no embedding multiplier, a layer without feed-forward
     "c": (config(130, 96, [

@@ -143,13 +143,29 @@ def gla_recurrence(q, k, v, alpha, state=None):
     return o, S
 
 
-def gla_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: float) -> torch.Tensor:
+def gla_cancellation(q, k, v, alpha) -> torch.Tensor:
+    """[n]: over the heads the smallest |o_t| / (|q_t| |S_t|), how much of the state's size survives the sum over key
+    channels.  The head norm divides by |o_t|: where almost everything cancels (the first token of a sequence whose
+    query is nearly orthogonal to its key, say) a rounding of q or k decides the output's sign."""
+    n, H, dk = q.shape
+    S = torch.zeros(H, dk, v.shape[-1], dtype=q.dtype)
+    out = torch.zeros(n, dtype=q.dtype)
+    for t in range(n):
+        S = alpha[t][:, :, None] * S + k[t][:, :, None] * v[t][:, None, :]
+        o = torch.einsum("hkv,hk->hv", S, q[t])
+        out[t] = (o.norm(dim=-1) / (q[t].norm(dim=-1) * S.flatten(1).norm(dim=-1) + 1e-300)).min()
+    return out
+
+
+def gla_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: float, cancel_out: Optional[List] = None) -> torch.Tensor:
     n = h.shape[0]
     H, dk, dv = m["heads"], m["dim"], m["vdim"]
     q = (h @ w["q"].T).view(n, H, dk) * dk ** -0.5
     k = (h @ w["k"].T).view(n, H, dk)
     v = (h @ w["v"].T).view(n, H, dv)
     o, _ = gla_recurrence(q, k, v, gla_decay(h, w, m))
+    if cancel_out is not None:
+        cancel_out.append(gla_cancellation(q, k, v, gla_decay(h, w, m)))
     o = rms_norm(o, w["norm"], eps).reshape(n, H * dv)          # every head by itself, one weight for all heads
     return (o * silu(h @ w["g"].T)) @ w["o"].T
 
@@ -229,7 +245,9 @@ def sub(tensors: Dict[str, torch.Tensor], prefix: str) -> Dict[str, torch.Tensor
 def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.float64, layers_out: Optional[List] = None,
             margins_out: Optional[List] = None):
     """Logits [n, vocab] of a whole sequence from position 0.  ``layers_out``: a list that gets the residual stream
-    after every layer; ``margins_out``: one that gets ``route_margin`` of every routed layer."""
+    after every layer; ``margins_out``: one that gets ``route_margin`` of every routed layer and four times
+    ``gla_cancellation`` of every recurrent layer (a value below about 0.08 of either kind: rounding to bfloat16 may
+    decide what the position computes)."""
     t = {k: v.to(dtype) if v.is_floating_point() else v for k, v in tensors.items()}
     ids = torch.as_tensor(list(tokens), dtype=torch.long)
     n = len(ids)
@@ -250,7 +268,10 @@ def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.
                 k, v = kept[i] = attention_keys_values(h1, w, m, positions)
             a = attention_mixer(h1, w, m, k, v, positions)
         elif layer["type"] == "gla":
-            a = gla_mixer(h1, w, m, eps)
+            cancel = [] if margins_out is not None else None
+            a = gla_mixer(h1, w, m, eps, cancel)
+            if cancel:
+                margins_out.append(4.0 * cancel[0])
         else:
             raise ValueError(layer["type"])
         f = layer.get("mlp")

@@ -84,8 +84,8 @@ def test_routing_by_hand():
     h, router = torch.ones(1, 1, dtype=torch.float64), z.T.clone()
     chosen, w = P.route(h, router, None, 2, 1.0)
     assert chosen.tolist() == [[3, 2]] and torch.allclose(w, torch.tensor([[4 / 7, 3 / 7]], dtype=torch.float64))
-    chosen, w = P.route(h, router, torch.tensor([0.25, 0.0, 0.0, 0.0], dtype=torch.float64), 2, 1.5)
-    assert chosen.tolist() == [[3, 0]] and torch.allclose(w, torch.tensor([[1.2, 0.3]], dtype=torch.float64))
+    chosen, w = P.route(h, router, torch.tensor([0.25, 0.0, 0.0, 0.0], dtype=torch.float64), 2, 2.5)
+    assert chosen.tolist() == [[3, 0]] and torch.allclose(w, torch.tensor([[2.0, 0.5]], dtype=torch.float64))
     # pass-through outputs hand the input on
     f = {"kind": "moe", "expert": {"ff": 2}, "router": {"experts": 1, "top": 1, "identity": 1, "scale": 2.0}}
     w = {"router": torch.tensor([[-5.0], [5.0]], dtype=torch.float64), "e0.gate": torch.ones(2, 1, dtype=torch.float64),
@@ -147,7 +147,7 @@ def test_the_configuration_refuses_what_it_cannot_run():
 def test_scaled_frequencies_of_the_engine_equal_the_plain_ones():
     from pico_vllm_amd.parts.rotary import scaled_frequencies
     for r in ({"dims": 16, "base": 10000.0, "scaling": dict(zip(("factor", "original", "fast", "slow"), YARN))},
-              {"dims": 64, "base": 500000.0}, {"dims": 32, "base": 1000.0, "scaling": {"factor": 8.0, "original": 32, "fast": 4.0, "slow": 0.5}}):
+              {"dims": 64, "base": 300000.0}, {"dims": 32, "base": 1000.0, "scaling": {"factor": 8.0, "original": 32, "fast": 4.0, "slow": 0.5}}):
         sc = r.get("scaling")
         f, mag = scaled_frequencies(r["dims"], r["base"], (sc["factor"], sc["original"], sc["fast"], sc["slow"]) if sc else None)
         pf, pmag = P.rotation_frequencies(r)
