@@ -63,9 +63,10 @@ class AttentionConfig:
     keep_first: int
     rot: Optional[RotationConfig]
     kv_from: Optional[int]
+    gated: bool = True     # False: a checkpoint without the gate's matrix
 
     @classmethod
-    def from_dict(cls, d: Dict[str, Any], where: str) -> "AttentionConfig":
+    def from_dict(cls, d: Dict[str, Any], where: str, gated: bool = True) -> "AttentionConfig":
         mask = d.get("mask") or {}
         dim = _int(d, "dim", where)
         kv_from = d.get("kv_from")
@@ -75,7 +76,8 @@ class AttentionConfig:
                   scale=_num(d, "scale", where), softcap=_num(d, "softcap", where) if d.get("softcap") is not None else 0.0,
                   window=_int(mask, "size", where + ".mask") if mask.get("size") is not None else 0,
                   keep_first=_int(mask, "keep_first", where + ".mask", least=0) if mask.get("keep_first") is not None else 0,
-                  rot=RotationConfig.from_dict(d["rot"], where + ".rot", dim) if d.get("rot") else None, kv_from=kv_from)
+                  rot=RotationConfig.from_dict(d["rot"], where + ".rot", dim) if d.get("rot") else None, kv_from=kv_from,
+                  gated=gated)
         if cfg.heads % cfg.kv_heads:
             raise ConfigError(f"{where}: {cfg.heads} heads are not a multiple of {cfg.kv_heads} kv_heads")
         if cfg.softcap < 0:
@@ -109,9 +111,10 @@ class FeedForwardConfig:
     identity: int = 0
     scale: float = 1.0
     shared_ff: int = 0     # 0: no shared expert
+    correction: bool = True    # False: a checkpoint without the choice's correction vector
 
     @classmethod
-    def from_dict(cls, d: Dict[str, Any], where: str) -> "FeedForwardConfig":
+    def from_dict(cls, d: Dict[str, Any], where: str, correction: bool = True) -> "FeedForwardConfig":
         kind = d.get("kind")
         if kind == "dense":
             return cls("dense", _int(d, "ff", where))
@@ -121,7 +124,7 @@ class FeedForwardConfig:
                       _int(ro, "top", where + ".router"),
                       _int(ro, "identity", where + ".router", least=0) if ro.get("identity") is not None else 0,
                       _num(ro, "scale", where + ".router") if ro.get("scale") is not None else 1.0,
-                      _int(sh, "ff", where + ".shared") if sh else 0)
+                      _int(sh, "ff", where + ".shared") if sh else 0, correction)
             if cfg.top > cfg.experts + cfg.identity:
                 raise ConfigError(f"{where}: top {cfg.top} of {cfg.experts + cfg.identity} router outputs")
             return cfg
@@ -155,8 +158,10 @@ class NasedraConfig:
             where = f"layers[{i}]"
             if not isinstance(l.get("mixer"), dict):
                 raise ConfigError(f"{where} lacks 'mixer'")
+            # tensors that a checkpoint may leave out (a gate, a correction of the choice) are taken as it has them
+            has = (lambda name: True) if shapes is None else (lambda name: name in shapes)
             if l.get("type") == "attention":
-                mixer = AttentionConfig.from_dict(l["mixer"], where + ".mixer")
+                mixer = AttentionConfig.from_dict(l["mixer"], where + ".mixer", gated=has(f"l{i}.mix.g"))
             elif l.get("type") == "gla":
                 # the inner size of the decay's matrices: the checkpoint's shape; else a key of the mixer (a model that
                 # is yet to be written); else the usual one
@@ -171,7 +176,8 @@ class NasedraConfig:
             else:
                 raise ConfigError(f"{where}: mixer type {l.get('type')!r} is not known (attention, gla)")
             mlp = l.get("mlp")
-            layers.append(NasedraLayer(l["type"], mixer, FeedForwardConfig.from_dict(mlp, where + ".mlp") if mlp else None))
+            layers.append(NasedraLayer(l["type"], mixer,
+                                       FeedForwardConfig.from_dict(mlp, where + ".mlp", has(f"l{i}.mlp.correction")) if mlp else None))
         for i, l in enumerate(layers):
             if l.type != "attention" or l.mixer.kv_from is None:
                 continue
@@ -214,6 +220,7 @@ def nasedra_spec(cfg: NasedraConfig) -> ModelSpec:
             mixer = PartSpec("gated_attention", {
                 "hidden_size": cfg.width, "num_heads": m.heads, "num_kv_heads": m.kv_heads, "key_dim": m.dim,
                 "value_dim": m.vdim, "scale": m.scale, "softcap": m.softcap, "window": m.window, "keep_first": m.keep_first,
+                "gated": m.gated,
                 "position": position, "own_kv": m.kv_from is None, "cache_window": cache_window,
                 "cache_keep_first": cache_keep})
             run_order.append(RunEntry(i, cache_of=m.kv_from))
@@ -230,7 +237,8 @@ def nasedra_spec(cfg: NasedraConfig) -> ModelSpec:
         else:
             ff = PartSpec("softmax_routed_experts", {
                 "hidden_size": cfg.width, "expert_size": l.mlp.ff, "num_experts": l.mlp.experts, "top": l.mlp.top,
-                "identity": l.mlp.identity, "scale": l.mlp.scale, "shared_size": l.mlp.shared_ff})
+                "identity": l.mlp.identity, "scale": l.mlp.scale, "shared_size": l.mlp.shared_ff,
+                "correction_name": "correction" if l.mlp.correction else None})
         layers.append(LayerSpec(prefix=f"l{i}", block="parallel_two_norms",
                                 slots={"norm1": ("norm1", norm), "mixer": ("mix", mixer), "norm2": ("norm2", norm),
                                        "ff": ("mlp", ff)}))

@@ -175,3 +175,15 @@ def test_pages_of_the_kept_first_positions_stay_when_the_window_passes():
     m.free_request("r")
     m.check()
     assert m.num_free_pages() == 12
+
+
+def test_a_checkpoint_without_gates_and_corrections_is_described_without_them():
+    from nasedra_configs import write_model
+    from pico_vllm_amd.config.registry import load_model_description
+    from pico_vllm_amd.parts.model import model_param_specs
+    cfg, _ = CONFIGS["a"]
+    kept = {k: v for k, v in tensors_of("a").items()
+            if not k.endswith(".correction") and not (k.endswith(".mix.g") and k.split(".")[0] in ("l0", "l2"))}
+    _, typed, spec = load_model_description(write_model(cfg, kept))
+    assert {p.name for p in model_param_specs(spec)} == set(kept)
+    assert not typed.layers[0].mixer.gated and not typed.layers[1].mlp.correction
