@@ -591,3 +591,52 @@ def test_greedy_generation_through_the_entry_point(dtype, graphs):
             assert float(logits[tok]) >= float(logits.max()) - slack, (dtype, p, o.token_ids, tok, int(logits.argmax()))
             toks.append(tok)
     llm.engine.runner.manager.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_replay_program_in_a_subprocess(dtype):
+    """bin/trace_run on a model folder of this design: steps on standard input, logits in files, `done` lines."""
+    import json
+    import os
+    import subprocess
+    import tempfile
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    name = "a"
+    reqs = requests(name, [40, 23, 31], seed=8)
+    steps = []
+    for rid, toks in reqs.items():           # r0 alone in portions; then the next, so that its pages and slot come back
+        parts = cut(toks, [9, 2, 14], tail=5)
+        at = 0
+        for i, n in enumerate(parts):
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[at:at + n], "want": list(range(n))}],
+                          "end": [rid] if i == len(parts) - 1 else []})
+            at += n
+    with tempfile.TemporaryDirectory() as out:
+        r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", model_dir(name), "--dtype", dtype, "--out", out,
+                            "--max-tokens", "64"], input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True,
+                           text=True, timeout=600)
+        assert r.returncode == 0, r.stderr[-2000:]
+        assert r.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+        rows, fed = {}, {}
+        for s in steps:
+            e = s["entries"][0]
+            a = np.fromfile(os.path.join(out, f"{s['step']}.f32"), dtype="<f4").reshape(len(e["want"]), -1)
+            for w, row in zip(e["want"], a):
+                rows[(e["id"], fed.get(e["id"], 0) + w)] = row
+            fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
+    compare(name, dtype, rows, reqs)
+
+
+def test_the_command_line_on_a_model_folder_of_this_design(capsys):
+    from pico_vllm_amd import run
+    assert run.main(["--model", model_dir("d"), "--prompt-ids", "5,17,3", "--prompt-ids", "9", "--max-new-tokens", "6",
+                     "--ignore-eos", "--dtype", "float32", "--num-gpu-blocks", "16", "--max-seq-len", "64"]) == 0
+    lines = [l for l in capsys.readouterr().out.splitlines() if l.startswith("[")]
+    assert len(lines) == 2 and all("(length)" in l and len(l.split(")")[1].split()) == 6 for l in lines)
+    cfg, t = CONFIGS["d"][0], tensors_of("d")
+    for line, prompt in zip(lines, ([5, 17, 3], [9])):
+        toks = list(prompt)
+        for tok in (int(x) for x in line.split(")")[1].split()):
+            logits = P.forward(cfg, t, toks)[-1]
+            assert float(logits[tok]) >= float(logits.max()) - 1e-4
+            toks.append(tok)
