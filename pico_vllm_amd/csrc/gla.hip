@@ -50,8 +50,9 @@ extern "C" int pico_gla_decay(const void* x, int ldx, int dtype, const void* a2,
 }
 
 // ---------------------------------------------------------------------------
-// The recurrence, token by token.  grid (sequences, heads, ceil(dv / 64)); a workgroup owns 64 value channels of one
-// head of one sequence; wave w of its ceil(dk / GLA_CPT) waves owns key channels GLA_CPT w .., lane l value channel l:
+// The recurrence, token by token.  grid (sequences, heads, ceil(dv / 64 VPL)); a workgroup owns 64 VPL value channels of
+// one head of one sequence; wave w of its ceil(dk / GLA_CPT) waves owns key channels GLA_CPT w .., lane l value channels
+// l, l + 64, .. (VPL of them: 2 where a head has more than 64):
 // a thread keeps GLA_CPT state elements in registers over all tokens of the step.  Tokens are taken TB (8 or 16) at a
 // time: their q, k and decays are staged in LDS (every thread reads all of its channels' from there) while the next
 // block's travel from memory in registers; the waves' partial outputs meet in LDS and are summed in wave order.
@@ -68,8 +69,9 @@ extern "C" int pico_gla_decay(const void* x, int ldx, int dtype, const void* a2,
 #define GLA_LOCAL 1
 #define GLA_FROM 2
 
-template <typename T, int MODE, int TB>
-__global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, int ldx, int q_col, int k_col, int v_col,
+// FUSED: the decays are made inside the walk (log_decay is null) instead of read.
+template <typename T, int MODE, int TB, int VPL, bool FUSED>
+__global__ __launch_bounds__(TB == 16 ? 256 : 512) void gla_scan_kernel(const T* __restrict__ x, int ldx, int q_col, int k_col, int v_col,
                                                        const float* __restrict__ log_decay,
                                                        const int* __restrict__ cu_seqlens,
                                                        const int* __restrict__ state_slots, float* __restrict__ state,
@@ -83,9 +85,18 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
   float* qs = lds;                                      // [TB][CP]
   float* ks = qs + TB * CP;
   float* as = ks + TB * CP;
-  float* po = as + TB * CP;                             // [TB][nw][64]
-  const int b = MODE == GLA_WHOLE ? blockIdx.x : blockIdx.x / max_chunks, h = blockIdx.y, v = blockIdx.z * 64 + lane;
-  const bool v_ok = v < dv;
+  float* po = as + TB * CP;                             // [TB][nw][64 VPL]
+  // a lane owns VPL value channels, 64 apart: what it reads of a token's q, k and decays out of LDS serves them all
+  // (every wave of a compute unit reads the same staged values, and LDS hands each lane its own copy)
+  constexpr int VW = 64 * VPL;
+  const int b = MODE == GLA_WHOLE ? blockIdx.x : blockIdx.x / max_chunks, h = blockIdx.y, v = blockIdx.z * VW + lane;
+  bool v_ok[VPL];
+  int v_in[VPL];                                        // a value channel that exists, else the head's last one
+#pragma unroll
+  for (int j = 0; j < VPL; j++) {
+    v_ok[j] = v + 64 * j < dv;
+    v_in[j] = min(v + 64 * j, dv - 1) - v;
+  }
   int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1];
   if (MODE != GLA_WHOLE) {
     t_begin += (blockIdx.x % max_chunks) * chunk;
@@ -96,9 +107,20 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
   const int c0 = wave * GLA_CPT;
   float* sp = MODE == GLA_WHOLE ? state + (((size_t)slot * H + h) * dk + c0) * dv + v
                                 : ws + (((size_t)blockIdx.x * H + h) * dk + c0) * dv + v;
-  float S[GLA_CPT];
+  // Every load below is unconditional, from an address clamped into the tensor, and what must not count is cleared
+  // afterwards: a load inside a branch is waited for inside that branch, and a thread's loads of a block then queue
+  // one behind the other's latency instead of travelling together.
+  float S[VPL][GLA_CPT];
+  if (MODE != GLA_LOCAL) {
 #pragma unroll
-  for (int c = 0; c < GLA_CPT; c++) S[c] = (MODE != GLA_LOCAL && v_ok && c0 + c < dk) ? sp[(size_t)c * dv] : 0.f;
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int c = 0; c < GLA_CPT; c++) S[j][c] = sp[(size_t)(min(c0 + c, dk - 1) - c0) * dv + v_in[j]];
+  }
+#pragma unroll
+  for (int j = 0; j < VPL; j++)
+#pragma unroll
+    for (int c = 0; c < GLA_CPT; c++) S[j][c] = (MODE != GLA_LOCAL && v_ok[j] && c0 + c < dk) ? S[j][c] : 0.f;
   if (MODE == GLA_LOCAL && blockIdx.z == 0) {
     // the chunk's decays multiplied up, as the sum of their logarithms, for the walk over the chunks
     for (int c = threadIdx.x; c < dk; c += blockDim.x) {
@@ -110,34 +132,36 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
   // A thread stages TB / 2 elements (token tt, channel c) of a block: i = threadIdx.x + j * blockDim.x.  The next
   // block's values travel in registers while this block is walked.
   constexpr int NL = TB / 2;
-  float rq[NL], rk[NL], ra[NL], rv[TB];
+  const int tt0 = (int)threadIdx.x >= CP ? 1 : 0, cc = (int)threadIdx.x - tt0 * CP;
+  T rq[NL], rk[NL], rv[VPL][TB];
+  float ra[NL];
+  const int c_in = min(cc, dk - 1);
   auto fetch = [&](int t0) {
     const int nb = min(TB, t_end - t0);
 #pragma unroll
     for (int j = 0; j < NL; j++) {
-      const int i = threadIdx.x + j * blockDim.x, tt = i / CP, c = i - tt * CP;
-      float qv = 0.f, kv = 0.f, av = 1.f;
-      if (tt < nb && c < dk) {
-        const T* row = x + (size_t)(t0 + tt) * ldx + (size_t)h * dk + c;
-        if (MODE != GLA_LOCAL) qv = load_f32(row + q_col) * qscale;
-        kv = load_f32(row + k_col);
-        if (log_decay) {
-          av = log_decay[(size_t)(t0 + tt) * H * dk + (size_t)h * dk + c];
-        } else {
-          // the decay's logarithm made here from the low-rank activations (as gla_decay_kernel does): one launch less
-          const T* xa = x + (size_t)(t0 + tt) * ldx + a_col;
-          const T* w = a2 + ((size_t)h * dk + c) * R;
-          float z = a2_bias ? a2_bias[h * dk + c] : 0.f;
-          for (int r = 0; r < R; r++) z = fmaf(load_f32(w + r), load_f32(xa + r), z);
-          const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
-          av = ls * inv_tau;
-        }
+      const int tt = min(tt0 + 2 * j, nb - 1);
+      const T* row = x + (size_t)(t0 + tt) * ldx + (size_t)h * dk + c_in;
+      rq[j] = MODE != GLA_LOCAL ? row[q_col] : row[k_col];
+      rk[j] = row[k_col];
+      if (!FUSED) {
+        ra[j] = log_decay[(size_t)(t0 + tt) * H * dk + (size_t)h * dk + c_in];
+      } else if (tt0 + 2 * j >= nb) {
+        ra[j] = 0.f;                                    // no such token in this block: nothing to work out
+      } else {
+        // the decay's logarithm made here from the low-rank activations (as gla_decay_kernel does): one launch less
+        const T* xa = x + (size_t)(t0 + tt) * ldx + a_col;
+        const T* w = a2 + ((size_t)h * dk + c_in) * R;
+        float z = a2_bias ? a2_bias[h * dk + c_in] : 0.f;
+        for (int r = 0; r < R; r++) z = fmaf(load_f32(w + r), load_f32(xa + r), z);
+        const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+        ra[j] = ls * inv_tau;
       }
-      rq[j] = qv; rk[j] = kv; ra[j] = av;
     }
 #pragma unroll
-    for (int tt = 0; tt < TB; tt++)
-      rv[tt] = (tt < nb && v_ok) ? load_f32(x + (size_t)(t0 + tt) * ldx + v_col + (size_t)h * dv + v) : 0.f;
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int tt = 0; tt < TB; tt++) rv[j][tt] = x[(size_t)(t0 + min(tt, nb - 1)) * ldx + v_col + (size_t)h * dv + v + v_in[j]];
   };
   fetch(t_begin);
   for (int t0 = t_begin; t0 < t_end; t0 += TB) {
@@ -145,14 +169,17 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
     __syncthreads();                                    // the last block's staged values and partial outputs have been read
 #pragma unroll
     for (int j = 0; j < NL; j++) {
-      const int i = threadIdx.x + j * blockDim.x, tt = i / CP, c = i - tt * CP;
-      qs[i] = rq[j];
-      ks[i] = rk[j];
-      as[i] = (tt < nb && c < dk) ? expf(ra[j]) : 1.f;
+      const int tt = tt0 + 2 * j, c = cc, i = tt * CP + c;      // = threadIdx.x + j * blockDim.x: a workgroup has 2 CP threads
+      const bool in = tt < nb && c < dk;
+      qs[i] = (in && MODE != GLA_LOCAL) ? load_f32(&rq[j]) * qscale : 0.f;
+      ks[i] = in ? load_f32(&rk[j]) : 0.f;
+      as[i] = in ? expf(ra[j]) : 1.f;
     }
-    float vv[TB];
+    float vv[VPL][TB];
 #pragma unroll
-    for (int tt = 0; tt < TB; tt++) vv[tt] = rv[tt];
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int tt = 0; tt < TB; tt++) vv[j][tt] = (tt < nb && v_ok[j]) ? load_f32(&rv[j][tt]) : 0.f;
     __syncthreads();
     if (t0 + TB < t_end) fetch(t0 + TB);
 #pragma unroll
@@ -161,38 +188,51 @@ __global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ x, 
       const float4* a4 = reinterpret_cast<const float4*>(as + tt * CP + c0);
       const float4* k4 = reinterpret_cast<const float4*>(ks + tt * CP + c0);
       const float4* q4 = reinterpret_cast<const float4*>(qs + tt * CP + c0);
-      float acc = 0.f;
+      // four partial sums over the channels (c mod 4), added at the end: four short chains instead of one long one
+      float acc0[VPL], acc1[VPL], acc2[VPL], acc3[VPL];
+#pragma unroll
+      for (int j = 0; j < VPL; j++) acc0[j] = acc1[j] = acc2[j] = acc3[j] = 0.f;
 #pragma unroll
       for (int c = 0; c < GLA_CPT / 4; c++) {
         const float4 av = a4[c], kv = k4[c];
-        S[4 * c + 0] = fmaf(av.x, S[4 * c + 0], kv.x * vv[tt]);
-        S[4 * c + 1] = fmaf(av.y, S[4 * c + 1], kv.y * vv[tt]);
-        S[4 * c + 2] = fmaf(av.z, S[4 * c + 2], kv.z * vv[tt]);
-        S[4 * c + 3] = fmaf(av.w, S[4 * c + 3], kv.w * vv[tt]);
-        if (MODE != GLA_LOCAL) {
-          const float4 qv = q4[c];
-          acc = fmaf(S[4 * c + 0], qv.x, acc);
-          acc = fmaf(S[4 * c + 1], qv.y, acc);
-          acc = fmaf(S[4 * c + 2], qv.z, acc);
-          acc = fmaf(S[4 * c + 3], qv.w, acc);
+        float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (MODE != GLA_LOCAL) qv = q4[c];
+#pragma unroll
+        for (int j = 0; j < VPL; j++) {
+          const float vt = vv[j][tt];
+          S[j][4 * c + 0] = fmaf(av.x, S[j][4 * c + 0], kv.x * vt);
+          S[j][4 * c + 1] = fmaf(av.y, S[j][4 * c + 1], kv.y * vt);
+          S[j][4 * c + 2] = fmaf(av.z, S[j][4 * c + 2], kv.z * vt);
+          S[j][4 * c + 3] = fmaf(av.w, S[j][4 * c + 3], kv.w * vt);
+          if (MODE != GLA_LOCAL) {
+            acc0[j] = fmaf(S[j][4 * c + 0], qv.x, acc0[j]);
+            acc1[j] = fmaf(S[j][4 * c + 1], qv.y, acc1[j]);
+            acc2[j] = fmaf(S[j][4 * c + 2], qv.z, acc2[j]);
+            acc3[j] = fmaf(S[j][4 * c + 3], qv.w, acc3[j]);
+          }
         }
       }
-      if (MODE != GLA_LOCAL) po[(tt * nw + wave) * 64 + lane] = acc;
+      if (MODE != GLA_LOCAL) {
+#pragma unroll
+        for (int j = 0; j < VPL; j++) po[(tt * nw + wave) * VW + 64 * j + lane] = (acc0[j] + acc1[j]) + (acc2[j] + acc3[j]);
+      }
     }
     if (MODE == GLA_LOCAL) continue;
     __syncthreads();
-    for (int i = threadIdx.x; i < nb * 64; i += blockDim.x) {
-      const int tt = i >> 6, l = i & 63, vo = blockIdx.z * 64 + l;
+    for (int i = threadIdx.x; i < nb * VW; i += blockDim.x) {
+      const int tt = i / VW, l = i % VW, vo = blockIdx.z * VW + l;
       if (vo >= dv) continue;
       float sum = 0.f;
-      for (int w = 0; w < nw; w++) sum += po[(tt * nw + w) * 64 + l];
+      for (int w = 0; w < nw; w++) sum += po[(tt * nw + w) * VW + l];
       out[(size_t)(t0 + tt) * H * dv + (size_t)h * dv + vo] = sum;
     }
   }
-  if (MODE != GLA_FROM && v_ok) {
+  if (MODE != GLA_FROM) {
 #pragma unroll
-    for (int c = 0; c < GLA_CPT; c++)
-      if (c0 + c < dk) sp[(size_t)c * dv] = S[c];
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int c = 0; c < GLA_CPT; c++)
+        if (v_ok[j] && c0 + c < dk) sp[(size_t)c * dv + 64 * j] = S[j][c];
   }
 }
 
@@ -244,18 +284,32 @@ extern "C" int pico_gla_scan(const void* x, int ldx, int dtype, int q_col, int k
   const int nw = (dk + GLA_CPT - 1) / GLA_CPT;
   // tokens of a block: 16 where the staged values fit (up to 128 key channels), else 8
   const int tb = nw <= 4 ? 16 : 8;
-  const size_t lds = (size_t)(3 * tb * nw * GLA_CPT + tb * nw * 64) * sizeof(float);
+  // value channels a lane: one.  (Two, where a head has more than 64, halve what is read out of LDS for the same
+  // arithmetic, but a wave then takes nearly twice as long and half as many fill the chip: 136 against 100 us for the
+  // chunks of a 2,048-token prompt with 12 heads of 64 x 128.)
+  const int vpl = 1;
+  const size_t lds = (size_t)(3 * tb * nw * GLA_CPT + tb * nw * 64 * vpl) * sizeof(float);
   PICO_REQUIRE(lds <= 64 * 1024, "pico_gla_scan: key channels beyond the staging memory");
-  const int vb = (dv + 63) / 64;
+  const int vb = (dv + 64 * vpl - 1) / (64 * vpl);
 #define GLA_ARGS(TT)                                                                                                       \
   (const TT*)x, ldx, q_col, k_col, v_col, log_decay, cu_seqlens, state_slots, state, out, H, dk, dv, qscale, num_slots,   \
       chunk, max_chunks, ws, ws_decay, (const TT*)a2, a2_bias, a_col, R, 1.0f / (tau > 0.f ? tau : 1.f)
 #define GLA_LAUNCH(TT, MODE, GX)                                                                                           \
   do {                                                                                                                     \
-    if (tb == 16)                                                                                                          \
-      gla_scan_kernel<TT, MODE, 16><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                              \
+    constexpr bool fused = MODE == GLA_WHOLE;     /* with FUSED the launch below is taken only when log_decay is null */ \
+    if (log_decay == nullptr && fused) {                                                                                   \
+      if (tb == 16)                                                                                                        \
+        gla_scan_kernel<TT, MODE, 16, 1, fused><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                  \
+      else                                                                                                                 \
+        gla_scan_kernel<TT, MODE, 8, 1, fused><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                   \
+    } else if (tb == 16 && vpl == 2)                                                                                       \
+      gla_scan_kernel<TT, MODE, 16, 2, false><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                    \
+    else if (tb == 16)                                                                                                     \
+      gla_scan_kernel<TT, MODE, 16, 1, false><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                    \
+    else if (vpl == 2)                                                                                                     \
+      gla_scan_kernel<TT, MODE, 8, 2, false><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                     \
     else                                                                                                                   \
-      gla_scan_kernel<TT, MODE, 8><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                               \
+      gla_scan_kernel<TT, MODE, 8, 1, false><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                     \
   } while (0)
 #define GLA_RUN(TT)                                                                                                        \
   if (chunk == 0) {                                                                                                        \
