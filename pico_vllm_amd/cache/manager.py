@@ -147,10 +147,10 @@ class CacheManager:
             if first_needed <= 0:
                 continue
             dead_upto = min(first_needed // self.page_size, len(rc.tables[gi]))
-            if rc.first_live[gi] == 0:
-                rc.first_live[gi] = min(_cdiv(g.keep_first, self.page_size), len(rc.tables[gi]))   # these pages stay
-            gone = [rc.tables[gi][j] for j in range(rc.first_live[gi], dead_upto)]
-            for j in range(rc.first_live[gi], dead_upto):
+            # pages 0 .. kept - 1 hold kept first positions and stay, whenever they were allocated
+            first = max(rc.first_live[gi], _cdiv(g.keep_first, self.page_size))
+            gone = [rc.tables[gi][j] for j in range(first, dead_upto)]
+            for j in range(first, dead_upto):
                 rc.tables[gi][j] = -1
             if gone:
                 g.pool.release(gone)

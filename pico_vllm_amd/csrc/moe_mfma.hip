@@ -280,7 +280,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const bf16_t* __restri
 #define MOE_FETCH(k0)                                                      \
   {                                                                        \
     const bool k_ok = (k0) + sk < K;                                       \
-    const int ko = k_ok ? (k0) : 0;                                        \
+    const int ko = k_ok ? (k0) : -sk;   /* the row's first 8, not 8 behind its end (the last row ends the tensor) */ \
     ra0 = *reinterpret_cast<const uint4*>(a_src0 + ko);                    \
     ra1 = *reinterpret_cast<const uint4*>(a_src1 + ko);                    \
     ra2 = *reinterpret_cast<const uint4*>(a_src2 + ko);                    \

@@ -40,14 +40,23 @@ def plain_logits(name, tokens):
     if key not in _plain:
         margins = []
         _plain[key] = P.forward(CONFIGS[name][0], tensors_of(name), tokens, margins_out=margins).numpy()
-        close = torch.stack(margins).min(0).values < CLOSE_CALL if margins else torch.zeros(len(tokens), dtype=torch.bool)
-        _plain[key + ("tainted",)] = (torch.cumsum(close.long(), 0) > 0).tolist()
+        least = torch.stack(margins).min(0).values if margins else torch.full((len(tokens),), float("inf"), dtype=torch.float64)
+        _plain[key + ("margin",)] = torch.cummin(least, 0).values.tolist()     # the smallest margin up to each position
     return _plain[key]
 
 
-def tainted(name, tokens, position):
+def margin_upto(name, tokens, position):
     plain_logits(name, tokens)
-    return _plain[(name, tuple(tokens), "tainted")][position]
+    return _plain[(name, tuple(tokens), "margin")][position]
+
+
+def tainted(name, tokens, position, close_call=CLOSE_CALL):
+    return margin_upto(name, tokens, position) < close_call
+
+
+# float32 rounds too: where a recurrent head's output cancels to less than half a percent of its state's size, the head
+# norm multiplies a rounding of 1e-7 by hundreds (seen at first tokens whose query is nearly orthogonal to their key)
+FLOAT32_CLOSE, FLOAT32_LOOSE = 0.02, 1e-3
 
 
 def replay(name, dtype, steps, max_tokens, page_size=16, max_live=4):
@@ -70,17 +79,20 @@ def replay(name, dtype, steps, max_tokens, page_size=16, max_live=4):
     return rows, rp
 
 
-def compare(name, dtype, rows, reqs):
+def compare(name, dtype, rows, reqs, bound=None, close_call=CLOSE_CALL):
+    bound = BOUND[dtype] if bound is None else bound
     errs = []
     for (rid, pos), got in rows.items():
         toks = reqs[rid.split("#")[0]]
         e = float(row_errors(got[None], plain_logits(name, toks)[pos][None])[0])
         errs.append(e)
-        if dtype == "bfloat16" and tainted(name, toks, pos):
+        if dtype == "bfloat16" and tainted(name, toks, pos, close_call):
             assert e <= TAINTED_BOUND, f"{name} {dtype}: {rid} position {pos}: {e:.3g}"
+        elif dtype == "float32" and tainted(name, toks, pos, FLOAT32_CLOSE):
+            assert e <= FLOAT32_LOOSE, f"{name} {dtype}: {rid} position {pos}: {e:.3g}"
         else:
-            assert e <= BOUND[dtype], f"{name} {dtype}: {rid} position {pos}: {e:.3g} > {BOUND[dtype]}"
-    assert np.median(errs) <= BOUND[dtype] / 2, f"{name} {dtype}: median {np.median(errs):.3g}"
+            assert e <= bound, f"{name} {dtype}: {rid} position {pos}: {e:.3g} > {bound}"
+    assert np.median(errs) <= bound / 2, f"{name} {dtype}: median {np.median(errs):.3g}"
 
 
 def requests(name, lengths, seed=0):
@@ -491,6 +503,36 @@ def test_experts_with_pass_through_outputs_and_a_shared_expert(dtype, E, ident, 
     assert err <= (1e-4 if dtype == "float32" else 6e-2) * max(1.0, float(want.abs().max())), err
 
 
+def mixed_steps(reqs, page, seed, max_live=3, tail=12):
+    """A schedule with at most ``max_live`` requests live: portions of changing size of some beside single tokens of
+    others (a request's last ``tail`` tokens go one by one), now and then a request left out of a step.  Returns the
+    steps and the most tokens that live requests held at any time, each request's count rounded up to whole pages."""
+    rng = random.Random(seed)
+    waiting, live, steps = list(reqs), {}, []
+    sizes = [17, 2, 40, 6, 29]
+    peak = 0
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            live[waiting.pop(0)] = 0
+        entries, end = [], []
+        for rid in list(live):
+            toks, at = reqs[rid], live[rid]
+            if rng.random() < 0.2 and len(live) > 1:
+                continue                                        # left out of this step
+            last = len(toks) - at <= tail
+            n = 1 if last else min(sizes[rng.randrange(len(sizes))], len(toks) - tail - at)
+            entries.append((rid, toks[at:at + n], range(n)))
+            live[rid] = at + n
+            if live[rid] == len(toks):
+                end.append(rid)
+        peak = max(peak, sum(roundup(live[r], page) for r in live))
+        for rid in end:
+            del live[rid]
+        if entries:
+            steps.append((entries, end))
+    return steps, roundup(peak)
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # whole models through the replayer
 # ---------------------------------------------------------------------------------------------------------------
@@ -532,30 +574,8 @@ def test_mixed_batches_in_a_pool_that_holds_what_is_live(name, dtype):
     just the live ones and with three state slots, so that pages and slots are used again; each request against itself alone."""
     lengths = [70, 33, 120, 9, 64, 47, 101]
     reqs = requests(name, lengths, seed=4)
-    rng = random.Random(7)
-    waiting, live, done_at, steps = list(reqs), {}, {}, []
-    sizes = [17, 2, 40, 6, 29]
-    peak = 0
-    while waiting or live:
-        while waiting and len(live) < 3:
-            live[waiting.pop(0)] = 0
-        entries, end = [], []
-        for rid in list(live):
-            toks, at = reqs[rid], live[rid]
-            if rng.random() < 0.2 and len(live) > 1:
-                continue                                        # left out of this step
-            tail = len(toks) - at <= 12
-            n = 1 if tail else min(sizes[rng.randrange(len(sizes))], len(toks) - 12 - at)
-            entries.append((rid, toks[at:at + n], range(n)))
-            live[rid] = at + n
-            if live[rid] == len(toks):
-                end.append(rid)
-        peak = max(peak, sum(roundup(live[r], PAGE[name]) for r in live))
-        for rid in end:
-            del live[rid]
-        if entries:
-            steps.append((entries, end))
-    rows, rp = replay(name, dtype, steps, roundup(peak), PAGE[name], max_live=3)
+    steps, peak = mixed_steps(reqs, PAGE[name], seed=7)
+    rows, rp = replay(name, dtype, steps, peak, PAGE[name], max_live=3)
     compare(name, dtype, rows, reqs)
     assert rp.runner.manager.num_free_pages() == rp.runner.manager.groups[0].pool.num_pages       # all given back
     if dtype == "float32":
@@ -640,3 +660,67 @@ def test_the_command_line_on_a_model_folder_of_this_design(capsys):
             logits = P.forward(cfg, t, toks)[-1]
             assert float(logits[tok]) >= float(logits.max()) - 1e-4
             toks.append(tok)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# configurations drawn at random
+# ---------------------------------------------------------------------------------------------------------------
+def draw_config(seed):
+    """Sizes, head counts, order of layers, masks, constants, feed-forwards: all drawn; returns (config, decay rank, page)."""
+    from nasedra_configs import attention, config, dense, gla, moe, rot
+    rng = random.Random(1000 + seed)
+    width = rng.choice([32, 40, 48, 64, 72, 96, 128])
+    layers, owners = [], []
+    for i in range(rng.randrange(2, 6)):
+        if rng.random() < 0.55:
+            mask = (None, None) if rng.random() < 0.2 else (rng.choice([1, 5, 16, 33, 64, 100]), rng.choice([None, 0, 1, 4, 17]))
+            cap = rng.choice([None, 8.0, 25.0, 60.0])
+            if owners and rng.random() < 0.35:
+                j = rng.choice(owners)
+                o = layers[j][0][1]
+                heads = o["kv_heads"] * rng.choice([1, 2, 3])
+                mixer = attention(heads, o["kv_heads"], o["dim"], o["vdim"], mask[0], mask[1], cap, o.get("rot"),
+                                  scale=o["dim"] ** -0.5 * rng.uniform(0.6, 1.4), kv_from=j)
+            else:
+                kv = rng.choice([1, 2, 4])
+                dim = rng.choice([8, 12, 16, 24, 32, 64])
+                r = None
+                if rng.random() < 0.85:
+                    scaling = None if rng.random() < 0.4 else (rng.choice([2.0, 4.0, 8.0]), rng.choice([16, 32, 64]),
+                                                               rng.choice([4.0, 8.0, 16.0]), rng.choice([0.5, 1.0, 2.0]))
+                    r = rot(rng.choice([x for x in (2, 4, 8, 12, 16, 32, 64) if x <= dim]), rng.choice([50.0, 1e4, 3e5]), scaling)
+                mixer = attention(kv * rng.choice([1, 2, 3, 5]), kv, dim, rng.choice([8, 16, 20, 32, 48]), mask[0], mask[1], cap, r,
+                                  scale=dim ** -0.5 * rng.uniform(0.6, 1.4))
+                owners.append(i)
+        else:
+            mixer = gla(rng.choice([1, 2, 3, 4]), rng.choice([8, 16, 24, 33, 48, 64, 80]), rng.choice([8, 16, 40, 64, 100]),
+                        rng.choice([1.0, 2.0, 8.0, 30.0]))
+        u = rng.random()
+        if u < 0.15:
+            ff = None
+        elif u < 0.55:
+            ff = dense(rng.choice([24, 40, 64, 100]))
+        else:
+            experts, ident = rng.randrange(2, 9), rng.choice([None, 0, 1, 3])
+            ff = moe(experts, rng.randrange(1, min(4, experts + (ident or 0)) + 1), rng.choice([16, 24, 32, 40]), ident,
+                     rng.choice([None, 0.6, 2.2]), rng.choice([None, 16, 40]))
+        layers.append((mixer, ff))
+    cfg = config(rng.randrange(40, 300), width, layers, eps=rng.choice([1e-5, 1e-6]), embed_scale=rng.choice([None, 0.5, 4.0]))
+    return cfg, rng.randrange(1, 9), rng.choice([8, 16, 32])
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_configurations_drawn_at_random_in_mixed_batches(seed):
+    import nasedra_configs as C
+    cfg, rank, page = draw_config(seed)
+    name = f"drawn{seed}"
+    C.CONFIGS[name] = (cfg, rank)
+    rng = random.Random(seed)
+    reqs = requests(name, [rng.randrange(1, 150) for _ in range(4)], seed=seed)
+    steps, peak = mixed_steps(reqs, page, seed=seed)
+    for dtype in ("float32", "bfloat16"):
+        rows, rp = replay(name, dtype, steps, peak, page, max_live=3)
+        # (widths down to 32 and heads of 8 channels: rounding to bfloat16 weighs three times what it does at the hand-made
+        # configurations' sizes; the float32 bound is the sharp one)
+        compare(name, dtype, rows, reqs, bound=None if dtype == "float32" else 3 * BOUND[dtype], close_call=0.25)
+        rp.runner.manager.check()

@@ -187,3 +187,25 @@ def test_a_checkpoint_without_gates_and_corrections_is_described_without_them():
     _, typed, spec = load_model_description(write_model(cfg, kept))
     assert {p.name for p in model_param_specs(spec)} == set(kept)
     assert not typed.layers[0].mixer.gated and not typed.layers[1].mlp.correction
+
+
+@pytest.mark.parametrize("window,keep,page,portions", [(1, 17, 16, [3, 1, 40, 2, 30, 1, 1, 50]), (1, 5, 4, [1] * 30), (7, 9, 8, [2, 2, 2, 60, 1, 1]),
+                                                       (3, 4, 4, [20, 1, 1, 1]), (16, 1, 16, [5, 100])])
+def test_kept_pages_stay_however_the_request_grows(window, keep, page, portions):
+    """The pages of the kept first positions may not exist yet when the window first passes a page: they stay all the same."""
+    from pico_vllm_amd.cache.manager import CacheManager
+    from pico_vllm_amd.parts.spec import CacheSpec, PageTensor
+    spec = CacheSpec("paged_kv", window=window, keep_first=keep, page_tensors=(PageTensor("k", (1, "page", 4)),))
+    m = CacheManager({0: spec}, page_size=page, num_pages=64, max_seqs=1)
+    assert m.add_request("r")
+    n = 0
+    for p in portions:
+        assert m.grow("r", n + p)
+        n += p
+        m.advance("r", n)
+        m.check()
+        table = m.block_table("r")
+        for j, pg in enumerate(table):
+            holds_kept = j * page < keep
+            readable = (j + 1) * page > n - window + 1          # the next query (position n) reads keys > n - window
+            assert (pg >= 0) == (holds_kept or readable), (n, j, table)
