@@ -724,3 +724,56 @@ def test_configurations_drawn_at_random_in_mixed_batches(seed):
         # configurations' sizes; the float32 bound is the sharp one)
         compare(name, dtype, rows, reqs, bound=None if dtype == "float32" else 3 * BOUND[dtype], close_call=0.25)
         rp.runner.manager.check()
+
+
+def draw_larger_config(seed):
+    """Sizes that the matrix-core kernels take (attention on the matrix cores, grouped experts, library products for long
+    portions): widths of 128 to 320, heads of 32 to 128 channels, up to 24 experts."""
+    from nasedra_configs import attention, config, dense, gla, moe, rot
+    rng = random.Random(5000 + seed)
+    width = rng.choice([128, 192, 256, 320])
+    layers, owners = [], []
+    for i in range(rng.randrange(3, 7)):
+        if rng.random() < 0.5:
+            mask = (None, None) if rng.random() < 0.15 else (rng.choice([17, 32, 64, 96, 128, 200]), rng.choice([None, 0, 2, 6, 16, 40]))
+            cap = rng.choice([None, 20.0, 50.0])
+            if owners and rng.random() < 0.4:
+                j = rng.choice(owners)
+                o = layers[j][0][1]
+                mixer = attention(o["kv_heads"] * rng.choice([1, 2, 4]), o["kv_heads"], o["dim"], o["vdim"], mask[0], mask[1], cap, o.get("rot"),
+                                  scale=o["dim"] ** -0.5 * rng.uniform(0.7, 1.3), kv_from=j)
+            else:
+                kv = rng.choice([1, 2, 4])
+                dim, vdim = rng.choice([(64, 64), (64, 96), (128, 64), (96, 48), (32, 96), (64, 32), (128, 128), (48, 64)])
+                scaling = None if rng.random() < 0.3 else (rng.choice([4.0, 8.0, 16.0]), rng.choice([64, 256, 1024]), rng.choice([8.0, 32.0]), rng.choice([1.0, 2.0]))
+                r = rot(rng.choice([x for x in (16, 32, 48, 64, 128) if x <= dim]), rng.choice([1e4, 5e5, 1e6]), scaling)
+                mixer = attention(kv * rng.choice([1, 2, 4, 6]), kv, dim, vdim, mask[0], mask[1], cap, r, scale=dim ** -0.5 * rng.uniform(0.7, 1.3))
+                owners.append(i)
+        else:
+            mixer = gla(rng.choice([2, 4, 6]), rng.choice([32, 48, 64, 128]), rng.choice([32, 64, 80, 128]), rng.choice([4.0, 16.0, 32.0]))
+        u = rng.random()
+        if u < 0.1:
+            ff = None
+        elif u < 0.5:
+            ff = dense(rng.choice([256, 320, 512]))
+        else:
+            experts, ident = rng.choice([4, 8, 16, 24]), rng.choice([None, 0, 2, 4])
+            ff = moe(experts, rng.randrange(1, 5), rng.choice([64, 96, 128]), ident, rng.choice([None, 1.5, 2.5]), rng.choice([None, 96, 128]))
+        layers.append((mixer, ff))
+    cfg = config(rng.randrange(300, 1000), width, layers, eps=1e-6, embed_scale=rng.choice([None, width ** 0.5]))
+    return cfg, rng.choice([8, 16, 32]), rng.choice([16, 16, 32])
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_larger_configurations_drawn_at_random_with_long_requests(seed):
+    import nasedra_configs as C
+    cfg, rank, page = draw_larger_config(seed)
+    name = f"larger{seed}"
+    C.CONFIGS[name] = (cfg, rank)
+    rng = random.Random(seed)
+    reqs = requests(name, [rng.randrange(150, 500) for _ in range(3)] + [rng.randrange(1, 40)], seed=seed)
+    steps, peak = mixed_steps(reqs, page, seed=seed, tail=40)
+    for dtype in ("float32", "bfloat16"):
+        rows, rp = replay(name, dtype, steps, peak, page, max_live=3)
+        compare(name, dtype, rows, reqs, close_call=0.25)
+        rp.runner.manager.check()
